@@ -6,7 +6,7 @@ with a softmax sink + dense / score-routed feed-forwards) on the same layer-list
 Framework layer: PyTorch-ROCm. Hot path: hand-written HIP kernels (``csrc/kernels``).
 Multi-GPU: one process per GPU, RCCL + a custom xGMI all-reduce. Decode: hipGraph replay.
 """
-from .config import LLaMAConfig, ModelArgs, ZasevikConfig, ZavevikConfig, config_from_params, get_preset, swiglu_hidden_size
+from .config import BesulixConfig, LLaMAConfig, ModelArgs, ZasevikConfig, ZavevikConfig, config_from_params, get_preset, swiglu_hidden_size
 from .generation import LLaMA
 from .models import (CausalLMOutput, FlaxLLaMAForCausalLM, FlaxLLaMAModel, KVCache, LLaMAForCausalLM,
                      LLaMAModel)
@@ -14,6 +14,7 @@ from .parallel.partition import (Mesh, P, PartitionSpec, get_llama_param_partiti
                                  with_named_sharding_constraint, with_sharding_constraint)
 from .models.registry import load_model
 from .models.zasevik import ZasevikForCausalLM
+from .models.besulix import BesulixForCausalLM
 from .models.zavevik import ZavevikForCausalLM
 from .runtime.engine import GenerationConfig
 from .runtime.stepper import SequenceStepper
@@ -28,5 +29,5 @@ __all__ = [
     "CausalLMOutput", "KVCache", "GenerationConfig",
     "Mesh", "P", "PartitionSpec", "get_llama_param_partition_spec", "with_named_sharding_constraint",
     "with_sharding_constraint", "LLaMA2Tokenizer", "LLaMA3Tokenizer", "ChatFormat", "convert_llama_weights",
-    "ZavevikConfig", "ZavevikForCausalLM", "ZasevikConfig", "ZasevikForCausalLM", "SequenceStepper", "load_model",
+    "ZavevikConfig", "ZavevikForCausalLM", "ZasevikConfig", "ZasevikForCausalLM", "BesulixConfig", "BesulixForCausalLM", "SequenceStepper", "load_model",
 ]

@@ -494,3 +494,172 @@ class ZasevikConfig:
 
     def __repr__(self) -> str:
         return f"ZasevikConfig {json.dumps(self.to_dict(), sort_keys=True)}"
+
+
+# -------------------------------------------------------------------------------------
+# Besulix: matrix-memory layers alternating with a chunked attention beside a time-mix recurrence
+# -------------------------------------------------------------------------------------
+@dataclass
+class MLSTMSpec:
+    """Matrix memory with exponential gates: ``heads`` heads of key size ``dim`` and value size ``vdim``; the gate
+    pre-activations are capped at ``gate_cap`` by a tanh."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+    type = "mlstm"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "MLSTMSpec":
+        heads, dim = int(d["heads"]), int(d["dim"])
+        return cls(heads=heads, dim=dim, vdim=int(d.get("vdim", dim)), gate_cap=float(d["gate_cap"]))
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(heads=self.heads, dim=self.dim, vdim=self.vdim, gate_cap=self.gate_cap)
+
+
+@dataclass
+class ChunkedAttentionSpec:
+    """Softmax attention with projection biases, rotary positions on the first ``rot_dims`` numbers of each q / k head
+    (and over the whole value head: values are cached rotated by their position and the sum is turned back), a
+    temperature and a sink per head, and a mask that keeps a query inside its block of ``chunk`` positions."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot_base: float
+    rot_dims: int
+    chunk: int
+    type = "chunked_attention"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "ChunkedAttentionSpec":
+        heads, dim = int(d["heads"]), int(d["dim"])
+        out = cls(heads=heads, kv_heads=int(d.get("kv_heads", heads)), dim=dim, vdim=int(d.get("vdim", dim)),
+                  scale=float(d["scale"]), rot_base=float(d["rot"]["base"]), rot_dims=int(d["rot"]["dims"]),
+                  chunk=int(d["mask"]["size"]))
+        if out.heads % out.kv_heads:
+            raise ValueError("heads must be divisible by kv_heads")
+        if out.rot_dims % 2 or out.rot_dims > out.dim or out.vdim % 2:
+            raise ValueError("rotary sizes: rot.dims even and at most dim, vdim even")
+        if out.chunk < 1:
+            raise ValueError("mask.size must be positive")
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(heads=self.heads, kv_heads=self.kv_heads, dim=self.dim, vdim=self.vdim, scale=self.scale,
+                    rot={"base": self.rot_base, "dims": self.rot_dims}, mask={"size": self.chunk})
+
+
+@dataclass
+class TimeMixSpec:
+    """Token-shifted linear recurrence with a decay per key channel: ``heads`` heads of size ``dim`` (keys and values)."""
+
+    heads: int
+    dim: int
+    type = "timemix"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "TimeMixSpec":
+        return cls(heads=int(d["heads"]), dim=int(d["dim"]))
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(heads=self.heads, dim=self.dim)
+
+
+@dataclass
+class ParallelSpec:
+    """Two mixers reading the same input; their outputs are summed with fixed weights."""
+
+    left: ChunkedAttentionSpec
+    right: TimeMixSpec
+    left_scale: float
+    right_scale: float
+    type = "parallel"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "ParallelSpec":
+        return cls(left=ChunkedAttentionSpec.from_dict(d["left"]), right=TimeMixSpec.from_dict(d["right"]),
+                   left_scale=float(d["left_scale"]), right_scale=float(d["right_scale"]))
+
+    def to_dict(self) -> Dict[str, Any]:
+        return dict(left=self.left.to_dict(), right=self.right.to_dict(), left_scale=self.left_scale,
+                    right_scale=self.right_scale)
+
+
+@dataclass
+class ClampedFFSpec:
+    """Dense gated feed-forward of width ``ff`` whose gate and up pre-activations are clamped at ``limit``."""
+
+    ff: int
+    limit: float
+    kind = "dense"
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"kind": "dense", "ff": self.ff, "limit": self.limit}
+
+
+class BesulixConfig:
+    """Besulix decoder: ``config.json`` with ``architecture: "Besulix"``, ``vocab``, ``width``, ``norm.eps``,
+    ``logit_softcap`` and a ``layers`` list of ``{type, mixer, mlp}`` entries; ``type`` is ``mlstm`` or ``parallel``,
+    ``mlp`` null or ``{kind: dense, ff, limit}``."""
+
+    model_type = "besulix"
+    architecture = "Besulix"
+    MIXERS = {"mlstm": MLSTMSpec, "parallel": ParallelSpec}
+
+    def __init__(self, vocab_size: int, hidden_size: int, layers, norm_eps: float = 1e-6, logit_softcap: float = 0.0,
+                 pad_token_id: int = -1, eos_token_id: Optional[int] = None):
+        self.vocab_size = int(vocab_size)
+        self.hidden_size = int(hidden_size)
+        self.layers = list(layers)
+        self.norm_eps = float(norm_eps)
+        self.logit_softcap = float(logit_softcap or 0.0)
+        self.pad_token_id = pad_token_id
+        self.eos_token_id = eos_token_id
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "BesulixConfig":
+        layers = []
+        for i, e in enumerate(d["layers"]):
+            if e["type"] not in cls.MIXERS:
+                raise ValueError(f"layer {i}: Besulix has no mixer {e['type']!r}")
+            f = e.get("mlp")
+            if f is not None and f.get("kind", "dense") != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f.get('kind')!r}")
+            layers.append(LayerSpec(cls.MIXERS[e["type"]].from_dict(e["mixer"]),
+                                    ClampedFFSpec(ff=int(f["ff"]), limit=float(f["limit"])) if f is not None else None))
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], layers=layers, norm_eps=d["norm"]["eps"],
+                   logit_softcap=d.get("logit_softcap", 0.0), pad_token_id=d.get("pad_token_id", -1),
+                   eos_token_id=d.get("eos_token_id"))
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+                "norm": {"eps": self.norm_eps}, "logit_softcap": self.logit_softcap,
+                "layers": [{"type": ls.mixer.type, "mixer": ls.mixer.to_dict(),
+                            "mlp": ls.mlp.to_dict() if ls.mlp is not None else None} for ls in self.layers]}
+
+    def save_pretrained(self, save_directory: str) -> None:
+        os.makedirs(save_directory, exist_ok=True)
+        with open(os.path.join(save_directory, "config.json"), "w") as f:
+            json.dump(self.to_dict(), f, indent=1, sort_keys=True)
+
+    @classmethod
+    def from_pretrained(cls, path: str) -> "BesulixConfig":
+        if os.path.isdir(path):
+            path = os.path.join(path, "config.json")
+        with open(path) as f:
+            return cls.from_dict(json.load(f))
+
+    def __eq__(self, other: object) -> bool:
+        return isinstance(other, BesulixConfig) and self.to_dict() == other.to_dict()
+
+    def __repr__(self) -> str:
+        return f"BesulixConfig {json.dumps(self.to_dict(), sort_keys=True)}"

@@ -106,6 +106,12 @@ class HybridCache:
       * ``("kv_from", j)``: no storage, ``layer(i)`` is layer ``j``'s keys and values (cross-layer KV sharing);
       * ``("delta", heads, kv_heads, dim, vdim, taps)``: a recurrent state ``[B, H, dim, vdim]`` (always fp32) and
         the short convolutions' input tail ``[B, 2 G dim + H vdim, taps - 1]`` (fp32);
+      * ``("mlstm", heads, dim, vdim)``: a matrix memory with its normaliser as one more value column
+        ``[B, H, dim, vdim + 1]`` and the running maximum of its gates ``[B, H]`` (fp32);
+      * ``("timemix", heads, dim, vdim, width)``: a matrix memory ``[B, H, dim, vdim]`` and the previous token's
+        mixer input ``[B, width]`` (fp32);
+      * ``("multi", spec, spec, ...)``: a layer whose mixers run side by side, each with its own entry (at most one
+        that holds keys and one that is recurrent);
       * ``None``: nothing.
     The slot index (tokens held, the same for every row) is mirrored on the device like ``KVCache``'s, so captured
     decode steps advance it without the host. ``dtype`` is the key / value element type (bf16, or fp32 for exact runs).
@@ -119,28 +125,51 @@ class HybridCache:
         self.dtype = dtype
         self._k, self._v, self._state, self._conv = {}, {}, {}, {}
         for i, sp in enumerate(self.specs):
-            if sp is None:
-                continue
-            if sp[0] == "kv":
-                _, g, dim, vdim = sp
-                self._k[i] = torch.zeros(batch_size, g, max_length, dim, dtype=dtype, device=device)
-                self._v[i] = torch.zeros(batch_size, g, max_length, vdim, dtype=dtype, device=device)
-            elif sp[0] == "latent":
-                self._k[i] = self._v[i] = torch.zeros(batch_size, 1, max_length, sp[1], dtype=dtype, device=device)
-            elif sp[0] == "kv_from":
-                j = sp[1]
-                if not (0 <= j < i) or self.specs[j] is None or self.specs[j][0] != "kv":
-                    raise ValueError(f"layer {i} shares the keys / values of layer {j}, which holds none before it")
-            elif sp[0] == "delta":
-                _, h, g, dim, vdim, taps = sp
-                self._state[i] = torch.zeros(batch_size, h, dim, vdim, dtype=torch.float32, device=device)
-                self._conv[i] = torch.zeros(batch_size, 2 * g * dim + h * vdim, max(taps - 1, 0),
-                                            dtype=torch.float32, device=device)
-            else:
-                raise ValueError(f"unknown cache spec {sp!r}")
+            for part in self.parts(sp):
+                self._alloc(i, part, batch_size, max_length, dtype, device)
         self._device = device
         self.index = 0
         self.index_t = torch.zeros(1, dtype=torch.int32, device=device)
+
+    @staticmethod
+    def parts(sp) -> list:
+        """The primitive entries of a layer's spec."""
+        if sp is None:
+            return []
+        if sp[0] == "multi":
+            kinds = [p[0] for p in sp[1:]]
+            if sum(k in ("kv", "latent", "kv_from") for k in kinds) > 1 or \
+                    sum(k in ("delta", "mlstm", "timemix") for k in kinds) > 1:
+                raise ValueError(f"a layer holds at most one key / value entry and one recurrent entry: {sp!r}")
+            return list(sp[1:])
+        return [sp]
+
+    def _alloc(self, i: int, sp, batch_size: int, max_length: int, dtype, device) -> None:
+        f32 = dict(dtype=torch.float32, device=device)
+        if sp[0] == "kv":
+            _, g, dim, vdim = sp
+            self._k[i] = torch.zeros(batch_size, g, max_length, dim, dtype=dtype, device=device)
+            self._v[i] = torch.zeros(batch_size, g, max_length, vdim, dtype=dtype, device=device)
+        elif sp[0] == "latent":
+            self._k[i] = self._v[i] = torch.zeros(batch_size, 1, max_length, sp[1], dtype=dtype, device=device)
+        elif sp[0] == "kv_from":
+            j = sp[1]
+            if not (0 <= j < i) or self.specs[j] is None or self.specs[j][0] != "kv":
+                raise ValueError(f"layer {i} shares the keys / values of layer {j}, which holds none before it")
+        elif sp[0] == "delta":
+            _, h, g, dim, vdim, taps = sp
+            self._state[i] = torch.zeros(batch_size, h, dim, vdim, **f32)
+            self._conv[i] = torch.zeros(batch_size, 2 * g * dim + h * vdim, max(taps - 1, 0), **f32)
+        elif sp[0] == "mlstm":
+            _, h, dim, vdim = sp
+            self._state[i] = torch.zeros(batch_size, h, dim, vdim + 1, **f32)
+            self._conv[i] = torch.zeros(batch_size, h, **f32)
+        elif sp[0] == "timemix":
+            _, h, dim, vdim, width = sp
+            self._state[i] = torch.zeros(batch_size, h, dim, vdim, **f32)
+            self._conv[i] = torch.zeros(batch_size, width, **f32)
+        else:
+            raise ValueError(f"unknown cache spec {sp!r}")
 
     @property
     def device(self):
@@ -148,15 +177,18 @@ class HybridCache:
 
     def layer(self, i: int):
         """Keys and values layer ``i`` attends over (its own, or the layer's it shares them with)."""
-        sp = self.specs[i]
-        j = sp[1] if sp[0] == "kv_from" else i
+        j = i
+        for part in self.parts(self.specs[i]):
+            if part[0] == "kv_from":
+                j = part[1]
         return self._k[j], self._v[j]
 
     def owns_kv(self, i: int) -> bool:
-        return self.specs[i] is not None and self.specs[i][0] == "kv"
+        return any(part[0] == "kv" for part in self.parts(self.specs[i]))
 
     def recurrent(self, i: int):
-        """``(state, conv tail)`` of a recurrent layer."""
+        """The two carried tensors of a recurrent layer: ``(state, convolution tail)`` (delta), ``(state with the
+        normaliser column, running maximum)`` (mlstm) or ``(state, previous token's input)`` (timemix)."""
         return self._state[i], self._conv[i]
 
     def advance(self, n: int) -> None:
@@ -188,16 +220,19 @@ class HybridCache:
         """Bytes a cache of this geometry takes (without allocating it)."""
         es = torch.empty(0, dtype=dtype).element_size()
         n = 0
-        for sp in specs:
-            if sp is None or sp[0] == "kv_from":
-                continue
-            if sp[0] == "kv":
-                n += batch_size * sp[1] * max_length * (sp[2] + sp[3]) * es
-            elif sp[0] == "latent":
-                n += batch_size * max_length * sp[1] * es
-            else:
-                _, h, g, dim, vdim, taps = sp
-                n += 4 * batch_size * (h * dim * vdim + (2 * g * dim + h * vdim) * max(taps - 1, 0))
+        for layer in specs:
+            for sp in HybridCache.parts(layer):
+                if sp[0] == "kv":
+                    n += batch_size * sp[1] * max_length * (sp[2] + sp[3]) * es
+                elif sp[0] == "latent":
+                    n += batch_size * max_length * sp[1] * es
+                elif sp[0] == "delta":
+                    _, h, g, dim, vdim, taps = sp
+                    n += 4 * batch_size * (h * dim * vdim + (2 * g * dim + h * vdim) * max(taps - 1, 0))
+                elif sp[0] == "mlstm":
+                    n += 4 * batch_size * sp[1] * (sp[2] * (sp[3] + 1) + 1)
+                elif sp[0] == "timemix":
+                    n += 4 * batch_size * (sp[1] * sp[2] * sp[3] + sp[4])
         return n
 
 

@@ -2,7 +2,7 @@
 ``models/mixers.py`` blocks shares -- the checkpoint directory round trip, the layered cache, and the step function
 ``forward_tokens`` that the generation engine (``runtime/engine.py``) and the request stepper (``runtime/stepper.py``)
 call. A family subclasses it with its configuration class, ``cache_specs`` and ``load_state_dict`` (which fills
-``embed``, ``blocks``, ``final_norm``, ``head`` and, if it has one, ``embed_scale``).
+``embed``, ``blocks``, ``final_norm``, ``head`` and, if it has them, ``embed_scale``, ``embed_norm``, ``logit_softcap``).
 
 Number formats: ``dtype=bfloat16`` (serving: bf16 matrix operands and caches, fp32 accumulation, and fp32 residual,
 norms, scores, recurrent state) or ``dtype=float32`` (everything exact fp32).
@@ -43,6 +43,8 @@ class LayerListLM:
         self.blocks: List = []
         self.embed: Optional[torch.Tensor] = None
         self.embed_scale = 1.0
+        self.embed_norm: Optional[torch.Tensor] = None  # fp32 [D]: gain of an RMS norm on the embedding
+        self.logit_softcap = 0.0                        # logits <- cap * tanh(logits / cap) when > 0
         self.final_norm: Optional[torch.Tensor] = None  # fp32 gain of the last norm: one number or [D]
         self.head: Optional[torch.Tensor] = None
         if _do_init:
@@ -62,12 +64,16 @@ class LayerListLM:
     def _weight_tensors(self) -> list:
         """Every tensor the model holds (for ``weight_bytes``)."""
         stack = [self.embed, self.head]
+
+        def walk(obj, depth):
+            for val in (vars(obj).values() if hasattr(obj, "__dict__") else obj if isinstance(obj, (list, tuple)) else ()):
+                if torch.is_tensor(val):
+                    stack.append(val)
+                elif val is not None and depth < 3 and (hasattr(val, "__dict__") or isinstance(val, (list, tuple))):
+                    walk(val, depth + 1)
+
         for blk in self.blocks:
-            for obj in vars(blk).values():
-                if torch.is_tensor(obj):
-                    stack.append(obj)
-                elif obj is not None and hasattr(obj, "__dict__"):
-                    stack += [t for t in vars(obj).values() if torch.is_tensor(t)]
+            walk(blk, 0)
         return stack
 
     # ------------------------------------------------------------------ checkpoints
@@ -120,6 +126,8 @@ class LayerListLM:
         idf = ids.reshape(-1).to(self.device, torch.int32).contiguous()
         ctx = StepContext(idf, positions.reshape(-1).to(self.device, torch.int32).contiguous(), b, s, cache, slot0)
         x = hy.embed_rows(idf, self.embed, scale=self.embed_scale)
+        if self.embed_norm is not None:
+            x = hy.rms_rows(x, self.embed_norm, self.eps)
         hidden = []
         for blk in self.blocks:
             blk(x, ctx)
@@ -135,7 +143,9 @@ class LayerListLM:
             xl = x
         else:
             raise ValueError(f"unknown logits_mode {logits_mode!r}")
-        logits = hy.linear(hy.rms_rows(xl, self.final_norm, self.eps), self.head)
+        cap = float(self.logit_softcap or 0.0)
+        logits = hy.linear(hy.rms_rows(xl, self.final_norm, self.eps), self.head,
+                           act=hy.ACT_SOFTCAP if cap > 0 else hy.ACT_NONE, limit=cap)
         return logits, x, hidden, []
 
     def gather_logits(self, logits_local: torch.Tensor) -> torch.Tensor:

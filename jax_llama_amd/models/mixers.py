@@ -16,6 +16,18 @@ the same mechanisms with other values.
   DenseFF         : dense feed-forward with a one-accumulator activation (squared ReLU).
   RoutedMoE       : sigmoid-score top-k router, input-weighted clamped-gate experts, gated shared expert.
   SandwichNormBlock : RMS norms on both sides of each sublayer, per-channel output gains.
+  RotaryChunkAttention : projection biases, rotary positions on part of each q / k head, values cached rotated by their
+                    position with the sum turned back, block-local causal mask, per-head temperature and sink.
+  MatrixLSTM      : matrix memory with capped exponential gates, a running maximum and a normaliser.
+  TimeMix         : token-shifted projections, per-channel decay from a low-rank map, bonus for the current token.
+  SideBySide      : several mixers on one input, their features concatenated in front of one output matrix.
+  GatedDenseFF    : dense feed-forward with a two-accumulator (gated) activation.
+  PreNormBlock    : ``x += sublayer(rms_norm(x))`` with the residual add in the output projection's epilogue.
+
+The blocks of the last group split a sublayer into ``features(h, ctx, out=None, gain=1.0)`` (everything up to the output
+projection; ``out`` a column slice to write into, ``gain`` a scalar folded into the last elementwise step) and the
+matrix ``w_o``, so a block can fuse the projection with the residual add and ``SideBySide`` can run one projection for
+all of its members.
 """
 from __future__ import annotations
 
@@ -247,3 +259,162 @@ class SandwichNormBlock:
         if self.mlp is not None:
             f = self.mlp(hy.RmsInput(x, self.pre2, self.eps), ctx)
             hy.norm_residual_(x, f.y, self.post2, self.eps, nsum=f.nsum, extra=f.extra, extra_gate=f.extra_gate)
+
+
+def _value(h):
+    return h.value() if isinstance(h, hy.RmsInput) else h
+
+
+class RotaryChunkAttention:
+    """Softmax attention over this layer's own keys and values with: one bias per projection column; rotary positions
+    on the first ``rot_dims`` numbers of every q / k head (number ``i`` paired with ``i + rot_dims / 2``); optionally
+    (``v_freq``) values rotated by their own position over the whole head before they are cached, and each head's summed
+    values turned back by the query's position; score ``q . k * scale * temp[h]``; optionally (``chunk``) a query sees
+    only the keys of its own block of ``chunk`` positions; optionally a learned sink per head in the denominator."""
+
+    def __init__(self, layer_idx: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, w_in: torch.Tensor,
+                 bias: Optional[torch.Tensor], qk_freq: torch.Tensor, v_freq: Optional[torch.Tensor],
+                 temp: Optional[torch.Tensor], sink: Optional[torch.Tensor], chunk: int, w_o: torch.Tensor):
+        self.i = layer_idx
+        self.heads, self.kv_heads, self.dim, self.vdim, self.scale = heads, kv_heads, dim, vdim, scale
+        self.w_in = w_in        # [H dim + G dim + G vdim, D]
+        self.bias = bias        # fp32 [H dim + G dim + G vdim] or None
+        self.qk_freq = qk_freq  # float64 [rot_dims / 2]
+        self.v_freq = v_freq    # float64 [vdim / 2] or None
+        self.temp, self.sink, self.chunk = temp, sink, chunk  # fp32 [H], fp32 [H], block length (0: causal only)
+        self.w_o = w_o          # [D, H vdim]
+        self.width = heads * vdim
+
+    def features(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None, gain: float = 1.0) -> torch.Tensor:
+        proj = hy.linear(h, self.w_in)
+        kc, vc = ctx.cache.layer(self.i)
+        q = hy.rope_prep(proj, self.bias, ctx.positions, ctx.slot0, ctx.b, ctx.s, self.heads, self.kv_heads, self.dim,
+                         self.vdim, kc, vc, self.qk_freq, self.v_freq)
+        a = hy.attn_bias(q, kc, vc, ctx.slot0, self.scale, sink=self.sink, chunk=self.chunk, head_scale=self.temp)
+        if self.v_freq is None and out is None and gain == 1.0:
+            return a
+        return hy.rotate_heads(a, ctx.positions, self.v_freq, self.heads, sign=-1.0, gain=gain, out=out)
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        return hy.linear(self.features(h, ctx), self.w_o)
+
+
+class MatrixLSTM:
+    """Matrix memory with exponential gates. Per head, with the capped gate pre-activations ``a`` (input) and ``f``
+    (log forget) and the running maximum ``m``: ``S <- e^(f + m' - m) S + e^(a - m) k v^T``, the normaliser ``z``
+    likewise with ``k`` alone, ``o = S^T q / (max(|z . q|, e^-m) + 1e-6)`` with ``q`` scaled by ``dim^-1/2``; then each
+    head's ``o`` over its root mean square, times a gain per column, times ``sigmoid(gate)``."""
+
+    def __init__(self, layer_idx: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float, w_in: torch.Tensor,
+                 gate_bias: torch.Tensor, norm_w: torch.Tensor, w_o: torch.Tensor):
+        self.i = layer_idx
+        self.heads, self.dim, self.vdim, self.cap, self.eps = heads, dim, vdim, gate_cap, eps
+        self.w_in = w_in            # [2 H dim + 2 H vdim + 2 H, D]: q | k | v | gate | input gate | forget gate
+        self.gate_bias = gate_bias  # fp32 [2 H]: input-gate biases, then forget-gate biases
+        self.norm_w = norm_w        # fp32 [H vdim]
+        self.w_o = w_o              # [D, H vdim]
+        self.width = heads * vdim
+
+    def features(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None, gain: float = 1.0) -> torch.Tensor:
+        nh, dim, vdim, m = self.heads, self.dim, self.vdim, ctx.b * ctx.s
+        proj = hy.linear(h, self.w_in)
+        state, mrun = ctx.cache.recurrent(self.i)
+        qk, vv = nh * dim, nh * vdim
+        keep, write, floor = hy.mlstm_prep(proj, 2 * qk + 2 * vv, 2 * qk + 2 * vv + nh, self.gate_bias, self.cap, mrun,
+                                           ctx.b, ctx.s, nh)
+        o = hy.mlstm_scan(proj[:, :qk].unflatten(1, (nh, dim)), proj[:, qk:2 * qk].unflatten(1, (nh, dim)),
+                          proj[:, 2 * qk:2 * qk + vv].unflatten(1, (nh, vdim)), keep, write, state, ctx.b, ctx.s,
+                          q_scale=dim ** -0.5)
+        return hy.gated_rmsnorm(o, proj[:, 2 * qk + vv:2 * qk + 2 * vv], self.norm_w, self.eps, hy.GATE_SIGMOID,
+                                denom_floor=floor, gain=gain, out=out)
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        return hy.linear(self.features(h, ctx), self.w_o)
+
+
+class TimeMix:
+    """Token-shifted linear recurrence. Each of the five projections reads its own blend of the current and the
+    previous token's input (``h + (h' - h) mu``); receptance, key, value per head; gate ``silu(.)``; a decay per key
+    channel ``exp(-exp(W_2 tanh(W_1 .) + w0))``; per head ``o = (S + diag(u) k v^T)^T r``, ``S <- diag(d) S + k v^T``;
+    then each head's ``o`` over its root mean square, times a gain per column, times the gate."""
+
+    def __init__(self, layer_idx: int, heads: int, dim: int, eps: float, mu: torch.Tensor, w_rkvg: torch.Tensor,
+                 w_d1: torch.Tensor, w_d2: torch.Tensor, w0: torch.Tensor, u: torch.Tensor, norm_w: torch.Tensor,
+                 w_o: torch.Tensor):
+        self.i = layer_idx
+        self.heads, self.dim, self.eps = heads, dim, eps
+        self.mu = mu          # fp32 [5, D]: blends of r, k, v, gate, decay
+        self.w_rkvg = w_rkvg  # [4, H dim, D]
+        self.w_d1, self.w_d2 = w_d1, w_d2  # [rank, D], [H dim, rank]
+        self.w0, self.u = w0, u            # fp32 [H, dim]
+        self.norm_w = norm_w  # fp32 [H dim]
+        self.w_o = w_o        # [D, H dim]
+        self.width = heads * dim
+
+    def features(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None, gain: float = 1.0) -> torch.Tensor:
+        nh, dim, m = self.heads, self.dim, ctx.b * ctx.s
+        state, prev = ctx.cache.recurrent(self.i)
+        mixes = hy.token_shift(_value(h), prev, self.mu, ctx.b, ctx.s)
+        if 4 * m <= hy.STACKED_MAX_ROWS:  # a few tokens: the four same-shaped projections as one grouped launch
+            r, k, v, g = hy.stacked_linear(mixes[:4], self.w_rkvg).unbind(0)
+        else:
+            r, k, v, g = (hy.linear(mixes[j], self.w_rkvg[j]) for j in range(4))
+        wpre = hy.linear(hy.linear(mixes[4], self.w_d1, act=hy.ACT_SOFTCAP, limit=1.0), self.w_d2)
+        hd = (nh, dim)
+        o = hy.timemix_scan(r.unflatten(1, hd), k.unflatten(1, hd), v.unflatten(1, hd), wpre.unflatten(1, hd), self.w0,
+                            self.u, state, ctx.b, ctx.s)
+        return hy.gated_rmsnorm(o, g, self.norm_w, self.eps, hy.GATE_SILU, gain=gain, out=out)
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        return hy.linear(self.features(h, ctx), self.w_o)
+
+
+class SideBySide:
+    """Mixers that read the same input; the result is ``sum_k scale_k * mixer_k(h)``. Their features are written side by
+    side (each scaled by its weight in its last elementwise step) and multiplied by the members' output matrices laid
+    side by side: one projection for all of them."""
+
+    def __init__(self, members, scales):
+        self.members, self.scales = list(members), [float(x) for x in scales]
+        self.w_o = torch.cat([mm.w_o for mm in self.members], 1).contiguous()
+        self.width = sum(mm.width for mm in self.members)
+
+    def features(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None, gain: float = 1.0) -> torch.Tensor:
+        hv = _value(h)
+        if out is None:
+            out = torch.empty(ctx.b * ctx.s, self.width, dtype=torch.float32, device=hv.device)
+        c = 0
+        for mm, sc in zip(self.members, self.scales):
+            mm.features(hv, ctx, out=out[:, c:c + mm.width], gain=gain * sc)
+            c += mm.width
+        return out
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        return hy.linear(self.features(h, ctx), self.w_o)
+
+
+class GatedDenseFF:
+    """``W_down act(W_gate h, W_up h)`` with a two-accumulator activation (the clamped gate by default:
+    ``g' sigmoid(alpha g') (u' + 1)``, ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)``)."""
+
+    def __init__(self, w_gu: torch.Tensor, w_down: torch.Tensor, limit: float, alpha: float, act: int = hy.ACT_CLAMP_GLU):
+        self.w_gu, self.w_o, self.limit, self.alpha, self.act = w_gu, w_down, limit, alpha, act
+
+    def features(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None, gain: float = 1.0) -> torch.Tensor:
+        return hy.linear(h, self.w_gu, act=self.act, limit=self.limit, alpha=self.alpha)
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        return hy.linear(self.features(h, ctx), self.w_o)
+
+
+class PreNormBlock:
+    """``x += mixer(norm1 * rms(x))``, ``x += ff(norm2 * rms(x))``: vector gains on the sublayers' inputs, the residual
+    add in the epilogue of each sublayer's output projection."""
+
+    def __init__(self, mixer, norm1: torch.Tensor, mlp, norm2: Optional[torch.Tensor], eps: float):
+        self.mixer, self.norm1, self.mlp, self.norm2, self.eps = mixer, norm1, mlp, norm2, eps
+
+    def __call__(self, x: torch.Tensor, ctx: StepContext) -> None:
+        hy.linear_add_(x, self.mixer.features(hy.RmsInput(x, self.norm1, self.eps), ctx), self.mixer.w_o)
+        if self.mlp is not None:
+            hy.linear_add_(x, self.mlp.features(hy.RmsInput(x, self.norm2, self.eps), ctx), self.mlp.w_o)

@@ -31,11 +31,17 @@ def _zasevik():
     return ZasevikConfig, ZasevikForCausalLM
 
 
+def _besulix():
+    from ..config import BesulixConfig
+    from .besulix import BesulixForCausalLM
+    return BesulixConfig, BesulixForCausalLM
+
+
 # architecture name (lower case) -> () -> (config class, model class)
 MODEL_REGISTRY: Dict[str, Callable[[], Tuple[type, type]]] = {"llama": _llama, "zavevik": _zavevik,
-                                                              "zasevik": _zasevik}
+                                                              "zasevik": _zasevik, "besulix": _besulix}
 # families on the layer-list step function (models/layer_list.py): both number formats, the hybrid extension
-LAYER_LIST_FAMILIES = ("zavevik", "zasevik")
+LAYER_LIST_FAMILIES = ("zavevik", "zasevik", "besulix")
 
 
 def register(name: str, factory: Callable[[], Tuple[type, type]]) -> None:

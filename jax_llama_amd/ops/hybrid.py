@@ -17,7 +17,14 @@ Mechanisms (each with its constants as arguments, usable by any model of the reg
     token is cached, queries are mapped into the latent space per head, every head attends over the shared latent
     (keys = values = the cache) with a learned sink in the softmax denominator, and the result is mapped out per head;
   * ``linear(act=...)``: squared-ReLU and clamped gated epilogues; ``moe_routed``: a sigmoid-score top-k router whose
-    weights scale the experts' INPUTS, plus a gated shared expert (``norm_residual_(extra=...)``).
+    weights scale the experts' INPUTS, plus a gated shared expert (``norm_residual_(extra=...)``);
+  * ``rope_prep`` / ``rotate_heads`` + ``attn_bias(chunk=..., head_scale=...)``: projection biases, rotary positions
+    on part of each q / k head, values rotated by their own position before caching and the summed values turned
+    back by the query's, block-local causal masks, a learned temperature per head;
+  * ``mlstm_prep`` / ``mlstm_scan`` and ``token_shift`` / ``timemix_scan``: two linear recurrences over a carried fp32
+    matrix state (a stabilised exponential-gate memory with a normaliser; a per-channel-decay memory with a bonus
+    for the current token), one scan kernel; ``gated_rmsnorm`` takes either's read-out;
+  * ``linear(act=ACT_SOFTCAP)`` and ``linear_add_``: ``cap * tanh(y / cap)`` epilogue; residual add in the epilogue.
 """
 from __future__ import annotations
 
@@ -34,7 +41,7 @@ F32 = torch.float32
 # widest key / value head the attention kernels take (csrc/hybrid/attn_bias.hip AB_MAX_DIM)
 ATTN_MAX_HEAD = 512
 # epilogues of a row linear (csrc/hybrid/hybrid.h RowAct)
-ACT_NONE, ACT_RELU2, ACT_SWIGLU, ACT_CLAMP_GLU = 0, 1, 2, 3
+ACT_NONE, ACT_RELU2, ACT_SWIGLU, ACT_CLAMP_GLU, ACT_SOFTCAP = 0, 1, 2, 3, 4
 
 _EXT = None
 _ERR: Optional[BaseException] = None
@@ -174,6 +181,8 @@ def _act_cpu(y: torch.Tensor, act: int, limit: float, alpha: float) -> torch.Ten
         return y
     if act == ACT_RELU2:
         return torch.relu(y).square()
+    if act == ACT_SOFTCAP:
+        return limit * torch.tanh(y / limit)
     n = y.shape[-1] // 2
     g, u = y[..., :n], y[..., n:]
     if act == ACT_SWIGLU:
@@ -184,7 +193,8 @@ def _act_cpu(y: torch.Tensor, act: int, limit: float, alpha: float) -> torch.Ten
 
 def linear(x, w: torch.Tensor, swiglu: bool = False, act: int = ACT_NONE, limit: float = 0.0,
            alpha: float = 1.0) -> torch.Tensor:
-    """``act(x [M, K] (fp32, or an ``RmsInput``) @ w^T)`` -> fp32 ``[M, N]``. ``act``: none, ``ACT_RELU2`` (``max(y, 0)^2``), or a gated
+    """``act(x [M, K] (fp32, or an ``RmsInput``) @ w^T)`` -> fp32 ``[M, N]``. ``act``: none, ``ACT_RELU2`` (``max(y, 0)^2``),
+    ``ACT_SOFTCAP`` (``limit * tanh(y / limit)``; ``limit = 1`` is a plain tanh), or a gated
     form for which ``w`` is ``[2N, K]`` (gate rows, then up rows): ``ACT_SWIGLU`` (``silu(g) * u``; also
     ``swiglu=True``) or ``ACT_CLAMP_GLU`` (``g' sigmoid(alpha g') (u' + 1)``, ``g' = min(g, limit)``,
     ``u' = clamp(u, -limit, limit)``). ``x`` may be a column-contiguous view with strided rows."""
@@ -203,6 +213,21 @@ def linear(x, w: torch.Tensor, swiglu: bool = False, act: int = ACT_NONE, limit:
     ext().linear_rows(x, None, w, out, None, None, None, x.shape[0], int(act), float(limit), float(alpha), None, norm_w,
                       norm_eps)
     return out
+
+
+def linear_add_(res: torch.Tensor, x, w: torch.Tensor) -> torch.Tensor:
+    """``res [M, N] (fp32) += x [M, K] @ w^T`` in place: a sublayer's output projection with the residual add in its
+    epilogue."""
+    x, norm_w, norm_eps = _fuse_norm(x, x.shape[0], w.shape[0])
+    if not _gpu(x):
+        return res.add_(_round_like(x, w) @ w.float().t())
+    if norm_w is None and res.is_contiguous() and _use_packed_gemm(x, w):
+        from . import linear_residual as packed_linear_residual
+        xb = torch.empty(x.shape, dtype=BF16, device=x.device)
+        ext().cast_bf16(x, xb)
+        return packed_linear_residual(xb, _packed_weight(w), res)
+    ext().linear_rows(x, None, w, res, None, None, None, x.shape[0], ACT_NONE, 0.0, 1.0, None, norm_w, norm_eps, 0, True)
+    return res
 
 
 _HEAD_INDEX = {}
@@ -240,6 +265,35 @@ def heads_linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         rows, offs = _head_index(m, h, x.device)
         e.linear_rows(x2, rows, w, out, rows, offs, None, m * h, ACT_NONE, 0.0, 1.0, None, None, 0.0, m)
     return out.reshape(m, h, n)
+
+
+# rows (members x tokens) up to which same-shaped projections of different inputs run as one grouped launch
+STACKED_MAX_ROWS = 64
+_STACK_INDEX = {}
+
+
+def stacked_linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """Same-shaped linears of different inputs in one launch: ``x [E, M, K]`` (fp32, contiguous), ``w [E, N, K]`` ->
+    fp32 ``[E, M, N]``, ``out[e] = x[e] @ w[e]^T``. Runs the expert-grouped row linear (member ``e`` = expert ``e``)."""
+    e_n, m, k = x.shape
+    n = w.shape[1]
+    if not _gpu(x):
+        return torch.einsum("emk,enk->emn", _round_like(x, w), w.float())
+    rows = e_n * m
+    out = torch.empty(rows, n, dtype=F32, device=x.device)
+    key = (e_n, m, str(x.device))
+    idx = _STACK_INDEX.get(key)
+    if idx is None:
+        if len(_STACK_INDEX) > 1024:
+            _STACK_INDEX.clear()
+        ar = torch.arange(e_n + 1, dtype=torch.int32)
+        idx = _STACK_INDEX[key] = (ar[:e_n].repeat_interleave(m).to(x.device), (ar * m).to(x.device))
+    ex = ext()
+    if rows <= ex.GEMV_MAX_R:
+        ex.linear_rows(x.reshape(rows, k), None, w, out, None, None, idx[0], rows, ACT_NONE, 0.0, 1.0, None, None, 0.0)
+    else:
+        ex.linear_rows(x.reshape(rows, k), None, w, out, None, idx[1], None, rows, ACT_NONE, 0.0, 1.0, None, None, 0.0, m)
+    return out.reshape(e_n, m, n)
 
 
 def moe_table(x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, w_gu: torch.Tensor,
@@ -492,11 +546,15 @@ def _expand_index(b: int, t: int, n: int, h: int, device):
 
 def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: float, softcap: float = 0.0,
               bias: Optional[torch.Tensor] = None, max_kv: Optional[int] = None,
-              sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+              sink: Optional[torch.Tensor] = None, chunk: int = 0,
+              head_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of ``q [B, S, H, dim]`` (queries at cache slots ``slot + s``) over ``[B, G, T, .]`` caches:
     ``score = q.k * scale``; ``softcap * tanh(score / softcap)`` if ``softcap > 0``; ``+ bias[min(i - j, last), h]``;
     softmax over ``j <= i``, with ``exp(sink[h])`` added to the denominator when ``sink [H]`` is given (a slot without
-    key or value). ``kc`` and ``vc`` may be one tensor (latent attention). Returns fp32 ``[B*S, H*vdim]``."""
+    key or value). ``chunk > 0``: query ``i`` only sees the keys of its own block of ``chunk`` cache slots,
+    ``floor(j / chunk) == floor(i / chunk)`` (blocks count from slot 0 of the row, wherever a prompt was cut).
+    ``head_scale [H]``: the score of head ``h`` is also multiplied by ``head_scale[h]`` (before cap and bias). ``kc`` and
+    ``vc`` may be one tensor (latent attention). Returns fp32 ``[B*S, H*vdim]``."""
     b, s, h, dim = q.shape
     g, vdim = kc.shape[1], vc.shape[3]
     if not _gpu(q):
@@ -505,6 +563,8 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
         k = kc[:, :, :t].float().repeat_interleave(h // g, 1)  # [B, H, t, dim]
         v = vc[:, :, :t].float().repeat_interleave(h // g, 1)
         sc = torch.einsum("bshd,bhtd->bhst", q.float(), k) * scale
+        if head_scale is not None:
+            sc = sc * head_scale.float().reshape(1, h, 1, 1)
         if softcap and softcap > 0:
             sc = softcap * torch.tanh(sc / softcap)
         qi = torch.arange(s0, t)[:, None]
@@ -513,7 +573,10 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
         if bias is not None:
             bt = bias.float()[dist.clamp(0, bias.shape[0] - 1)]  # [s, t, H]
             sc = sc + bt.permute(2, 0, 1)[None]
-        sc = sc.masked_fill((dist < 0)[None, None], float("-inf"))
+        hidden = dist < 0
+        if chunk and chunk > 0:
+            hidden = hidden | (torch.div(qi, chunk, rounding_mode="floor") != torch.div(kj, chunk, rounding_mode="floor"))
+        sc = sc.masked_fill(hidden[None, None], float("-inf"))
         if sink is not None:
             sc = torch.cat([sc, sink.float().reshape(1, h, 1, 1).expand(b, h, s, 1)], -1)
             pr = torch.softmax(sc, -1)[..., :-1]
@@ -526,14 +589,14 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
     t_cap = int(max_kv) if max_kv is not None else kc.shape[2]
     ws, splits, vt = None, 1, None
     if s == 1:
-        splits = int(e.attn_decode_splits(b, h, t_cap))
+        splits = int(e.attn_decode_splits(b, h, min(t_cap, chunk) if chunk and chunk > 0 else t_cap))
         ws = torch.empty(b * h * splits * (vdim + 2), dtype=F32, device=q.device)
     elif MMA_PREFILL:
         nb = int(e.attn_prefill_ws_bytes(b, s, g, dim, vdim, kc.shape[2], kc.dtype == BF16))
         if nb:  # bf16 caches at the MFMA shapes: the flash kernel over a transposed copy of the values
             vt = torch.empty(nb // 2, dtype=BF16, device=q.device)
     e.attn_bias(q.contiguous(), kc, vc, _slot_tensor(slot, q.device), float(scale), float(softcap or 0.0), bias, out,
-                t_cap, ws, splits, vt, sink)
+                t_cap, ws, splits, vt, sink, int(chunk or 0), head_scale)
     return out
 
 
@@ -605,13 +668,191 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Te
     return o
 
 
-def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    """``o [M, H, vdim] / rms(o) * w [vdim] * silu(gate [M, H*vdim])`` -> fp32 ``[M, H*vdim]``."""
-    m, h, vdim = o.shape
+GATE_SILU, GATE_SIGMOID = 0, 1
+
+
+def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float, gate_act: int = GATE_SILU,
+                  denom_floor: Optional[torch.Tensor] = None, gain: float = 1.0,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``o [M, H, vdim] / rms(o) * w * act(gate [M, H*vdim]) * gain`` -> fp32 ``[M, H*vdim]``. ``w``: ``[vdim]`` (one
+    gain vector for every head) or ``[H*vdim]``; ``gate_act``: ``GATE_SILU`` or ``GATE_SIGMOID``. ``denom_floor [M, H]``:
+    ``o`` is ``[M, H, vdim + 1]`` whose last column is a normaliser ``z``; the head's first ``vdim`` numbers are divided
+    by ``max(|z|, denom_floor) + 1e-6`` before the norm. ``out``: a ``[M, H*vdim]`` column slice of a wider buffer."""
+    m, h, ov = o.shape
+    vdim = ov - 1 if denom_floor is not None else ov
+    if out is None:
+        out = torch.empty(m, h * vdim, dtype=F32, device=o.device)
     if not _gpu(o):
         x = o.float()
-        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
-        return x.reshape(m, h * vdim) * torch.nn.functional.silu(gate.float())
-    out = torch.empty(m, h * vdim, dtype=F32, device=o.device)
-    ext().gated_rmsnorm(o, gate, w, float(eps), out, h, vdim)
+        if denom_floor is not None:
+            x = x[..., :vdim] / (torch.maximum(x[..., vdim].abs(), denom_floor.float().reshape(m, h)) + 1e-6)[..., None]
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        x = x.reshape(m, h * vdim) * (w.float().repeat(h) if w.numel() == vdim and h > 1 else w.float().reshape(-1))
+        g = gate.float()
+        out.copy_(x * (torch.sigmoid(g) if gate_act == GATE_SIGMOID else torch.nn.functional.silu(g)) * gain)
+        return out
+    ext().gated_rmsnorm(o, gate, w, float(eps), out, h, vdim, int(gate_act), denom_floor, float(gain))
     return out
+
+
+# ------------------------------------------------------------------------------------------------ rotary positions
+def rotary_freqs(base: float, dims: int, device) -> torch.Tensor:
+    """float64 ``[dims / 2]``: ``base^(-2 i / dims)``, the turn per position of pair ``i``. Angles are formed in 64-bit
+    (position times this) so that a position in the thousands keeps the sine's and cosine's full 32-bit accuracy."""
+    if dims < 0 or dims % 2:
+        raise ValueError(f"rotary dims must be even, got {dims}")
+    return torch.tensor([float(base) ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float64, device=device)
+
+
+def _turn_cpu(x: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, sign: float = 1.0) -> torch.Tensor:
+    """Rotate the first ``2 len(freq)`` numbers of the last axis of ``x [M, heads, n]`` by ``sign * pos[m]``: number
+    ``i`` pairs with ``i + len(freq)``."""
+    half = freq.numel()
+    if half == 0:
+        return x
+    ang = pos.reshape(-1).double()[:, None] * freq.double()[None, :] * sign
+    c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+    u, v = x[..., :half], x[..., half:2 * half]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * half:]], -1)
+
+
+def rope_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor, slot, b: int, s: int, heads: int,
+              kv_heads: int, dim: int, vdim: int, kc: torch.Tensor, vc: torch.Tensor, qk_freq: torch.Tensor,
+              v_freq: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From the fused projection ``proj [B*S, H*dim + G*dim + G*vdim]`` (+ ``bias``, one number per column): q and k
+    heads rotated by the token's position on their first ``2 len(qk_freq)`` numbers (number ``i`` with
+    ``i + len(qk_freq)``, angle ``position * qk_freq[i]``; the rest pass), v heads rotated the same way over
+    ``2 len(v_freq)`` numbers when ``v_freq`` is given; k / v written into the caches ``[B, G, T, .]`` at ``slot + s``.
+    Returns q ``[B, S, H, dim]`` fp32."""
+    m = b * s
+    if not _gpu(proj):
+        s0 = _slot_int(slot)
+        y = proj.float()
+        if bias is not None:
+            y = y + bias.float()
+        pos = positions.reshape(-1)
+        q = _turn_cpu(y[:, :heads * dim].reshape(m, heads, dim), pos, qk_freq)
+        k = _turn_cpu(y[:, heads * dim:(heads + kv_heads) * dim].reshape(m, kv_heads, dim), pos, qk_freq)
+        v = y[:, (heads + kv_heads) * dim:(heads + kv_heads) * dim + kv_heads * vdim].reshape(m, kv_heads, vdim)
+        if v_freq is not None:
+            v = _turn_cpu(v, pos, v_freq)
+        kc[:, :, s0:s0 + s] = k.reshape(b, s, kv_heads, dim).permute(0, 2, 1, 3).to(kc.dtype)
+        vc[:, :, s0:s0 + s] = v.reshape(b, s, kv_heads, vdim).permute(0, 2, 1, 3).to(vc.dtype)
+        return q.reshape(b, s, heads, dim).contiguous()
+    q = torch.empty(b, s, heads, dim, dtype=F32, device=proj.device)
+    ext().rope_prep(proj, bias, positions.reshape(-1).to(torch.int32).contiguous(), _slot_tensor(slot, proj.device), b, s,
+                    heads, kv_heads, dim, vdim, kc, vc, q, qk_freq, v_freq)
+    return q
+
+
+def rotate_heads(a: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], heads: int, sign: float = 1.0,
+                 gain: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out [M, heads * n] = turn(a [M, heads * n], sign * position) * gain``: every head's first ``2 len(freq)``
+    numbers rotated (pairs ``i``, ``i + len(freq)``) by ``sign`` times the row's position; ``freq`` None: a scaled copy.
+    ``out`` may be a column slice of a wider buffer."""
+    m = a.shape[0]
+    n = a.shape[1] // heads
+    if out is None:
+        out = torch.empty(m, heads * n, dtype=F32, device=a.device)
+    if not _gpu(a):
+        x = a.float().reshape(m, heads, n)
+        if freq is not None:
+            x = _turn_cpu(x, positions.reshape(-1), freq, sign)
+        out.copy_(x.reshape(m, heads * n) * gain)
+        return out
+    ext().rotate_heads(a, positions.reshape(-1).to(torch.int32).contiguous(), freq, heads, float(sign), float(gain), out)
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ linear recurrences
+def token_shift(h: torch.Tensor, prev: torch.Tensor, mu: torch.Tensor, b: int, s: int) -> torch.Tensor:
+    """``out[n, m] = h[m] + (h[m - 1] - h[m]) * mu[n]`` for the ``n`` rows of ``mu [n, D]``; the token before a call's
+    first comes from ``prev [B, D]`` (zeros at a sequence start), which is then set to the call's last token. fp32
+    ``[n, B*S, D]``."""
+    n, d = mu.shape
+    if not _gpu(h):
+        hh = h.float().reshape(b, s, d)
+        before = torch.cat([prev.float()[:, None], hh[:, :-1]], 1)
+        out = hh[None] + (before - hh)[None] * mu.float()[:, None, None, :]
+        prev.copy_(hh[:, -1])
+        return out.reshape(n, b * s, d).contiguous()
+    out = torch.empty(n, b * s, d, dtype=F32, device=h.device)
+    ext().token_shift(h, prev, mu, out, b, s)
+    return out
+
+
+def mlstm_prep(proj: torch.Tensor, col_i: int, col_f: int, gate_bias: torch.Tensor, cap: float, mstate: torch.Tensor,
+               b: int, s: int, heads: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gates of the stabilised exponential-gate memory from columns of ``proj [B*S, .]``: per head
+    ``a = cap tanh((proj[col_i + h] + gate_bias[h]) / cap)``, ``f = logsigmoid(cap tanh((proj[col_f + h] +
+    gate_bias[H + h]) / cap))``, the running maximum ``m_t = max(f + m_(t-1), a)`` carried in ``mstate [B, H]`` (0 at a
+    sequence start; advanced). Returns ``(keep, write, floor)`` fp32 ``[B*S, H]``: ``exp(f + m_(t-1) - m_t)``,
+    ``exp(a - m_t)``, ``exp(-m_t)``."""
+    m = b * s
+    if not _gpu(proj):
+        gb = gate_bias.float()
+        a = cap * torch.tanh((proj[:, col_i:col_i + heads].float() + gb[:heads]) / cap)
+        f = torch.nn.functional.logsigmoid(cap * torch.tanh((proj[:, col_f:col_f + heads].float() + gb[heads:]) / cap))
+        a, f = a.reshape(b, s, heads), f.reshape(b, s, heads)
+        keep, write, floor = torch.empty(b, s, heads), torch.empty(b, s, heads), torch.empty(b, s, heads)
+        mm = mstate.float().clone()
+        for t in range(s):
+            m_new = torch.maximum(f[:, t] + mm, a[:, t])
+            keep[:, t] = torch.exp(f[:, t] + mm - m_new)
+            write[:, t] = torch.exp(a[:, t] - m_new)
+            floor[:, t] = torch.exp(-m_new)
+            mm = m_new
+        mstate.copy_(mm)
+        return keep.reshape(m, heads), write.reshape(m, heads), floor.reshape(m, heads)
+    out = torch.empty(3, m, heads, dtype=F32, device=proj.device)
+    ext().mlstm_prep(proj, int(col_i), int(col_f), gate_bias, float(cap), mstate, out, b, s, heads)
+    return out[0], out[1], out[2]
+
+
+def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, keep: torch.Tensor, write: torch.Tensor,
+               state: torch.Tensor, b: int, s: int, q_scale: float = 1.0) -> torch.Tensor:
+    """Matrix memory with scalar gates per head, read after the write. ``q, k [M, H, dim]``, ``v [M, H, vdim]`` (column
+    views of a projection are fine), ``keep, write [M, H]``; ``state [B, H, dim, vdim + 1]`` (fp32, advanced), whose last
+    column is the normaliser (the memory of a value that is always 1):
+    ``S <- keep S + write k [v, 1]^T;  o = S^T (q_scale q)``. Returns ``o [M, H, vdim + 1]``."""
+    m, h, dim = q.shape
+    vdim = v.shape[2]
+    if not _gpu(q):
+        qq = q.float().reshape(b, s, h, dim) * q_scale
+        kk = k.float().reshape(b, s, h, dim)
+        vv = torch.cat([v.float().reshape(b, s, h, vdim), torch.ones(b, s, h, 1)], -1)
+        ke, wr = keep.float().reshape(b, s, h), write.float().reshape(b, s, h)
+        o = torch.empty(b, s, h, vdim + 1)
+        for t in range(s):
+            state.mul_(ke[:, t, :, None, None])
+            state.add_(wr[:, t, :, None, None] * kk[:, t, :, :, None] * vv[:, t, :, None, :])
+            o[:, t] = torch.einsum("bhdv,bhd->bhv", state, qq[:, t])
+        return o.reshape(m, h, vdim + 1)
+    o = torch.empty(m, h, vdim + 1, dtype=F32, device=q.device)
+    ext().lin_scan(0, q, k, v, keep, write, None, None, state, o, b, s, float(q_scale))
+    return o
+
+
+def timemix_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wpre: torch.Tensor, w0: torch.Tensor,
+                 u: torch.Tensor, state: torch.Tensor, b: int, s: int) -> torch.Tensor:
+    """Matrix memory with a decay per key channel and a bonus for the current token, read before the write.
+    ``r, k [M, H, dim]``, ``v [M, H, vdim]``, ``wpre [M, H, dim]`` (column views are fine), ``w0, u [H, dim]``;
+    ``state [B, H, dim, vdim]`` (fp32, advanced): ``d = exp(-exp(wpre + w0))``;
+    ``o = (S + diag(u) k v^T)^T r;  S <- diag(d) S + k v^T``. Returns ``o [M, H, vdim]``."""
+    m, h, dim = r.shape
+    vdim = v.shape[2]
+    if not _gpu(r):
+        rr, kk = r.float().reshape(b, s, h, dim), k.float().reshape(b, s, h, dim)
+        vv = v.float().reshape(b, s, h, vdim)
+        dd = torch.exp(-torch.exp(wpre.float().reshape(b, s, h, dim) + w0.float().reshape(h, dim)))
+        uu = u.float().reshape(h, dim)
+        o = torch.empty(b, s, h, vdim)
+        for t in range(s):
+            kv = kk[:, t, :, :, None] * vv[:, t, :, None, :]
+            o[:, t] = torch.einsum("bhdv,bhd->bhv", state + uu[None, :, :, None] * kv, rr[:, t])
+            state.mul_(dd[:, t, :, :, None])
+            state.add_(kv)
+        return o.reshape(m, h, vdim)
+    o = torch.empty(m, h, vdim, dtype=F32, device=r.device)
+    ext().lin_scan(1, r, k, v, wpre, None, w0.reshape(h, dim), u.reshape(h, dim), state, o, b, s, 1.0)
+    return o
