@@ -11,6 +11,9 @@
 // The bias table is indexed by distance (rows past the last repeat it), so any bucketing is a host-side table fill.
 // An optional per-head sink adds exp(sink[h]) to the softmax denominator: the running maximum starts at the sink and
 // the running sum at 1 (in decode, for the first key split only), so no kernel needs a branch per key for it.
+// Block-local masks (chunk > 0): a query at slot i sees the keys of [floor(i / chunk) * chunk, i]; every kernel starts
+// its key walk at that block's first slot, so the keys before it are never read. A per-head factor (head_scale) joins
+// the score scale.
 #include "hy_util.h"
 #include "hybrid.h"
 
@@ -91,6 +94,7 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
   const CT* vbase = reinterpret_cast<const CT*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.vdim;
   const bool fastk = (p.dim & 7) == 0 && ((uintptr_t)kbase & 15) == 0;
   const bool sunk = with_sink && p.sink;
+  const float hs = p.head_scale ? p.head_scale[h] : 1.f;
   m_run = sunk ? p.sink[h] : -INFINITY;
   l_run = sunk ? 1.f : 0.f;
 #pragma unroll
@@ -115,7 +119,7 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
       } else {
         for (int d = 0; d < p.dim; ++d) d0 = fmaf(qs[d], ab_ld(kr + d), d0);
       }
-      sc = (d0 + d1) * p.scale;
+      sc = (d0 + d1) * p.scale * hs;
       if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
       if (p.bias) sc += p.bias[(size_t)min(qi - j, p.nbias - 1) * p.H + h];
     }
@@ -148,6 +152,17 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
   }
 }
 
+// first key slot a query at slot qi sees
+JLA_DEV int ab_first_key(const AttnBias& p, int qi) { return p.chunk > 0 ? qi / p.chunk * p.chunk : 0; }
+
+// keys [j_lo, j_hi) of decode split sp: the query's visible keys [lo, qi] dealt to the splits in runs of 64
+JLA_DEV void ab_split_range(const AttnBias& p, int qi, int sp, int& j_lo, int& j_hi) {
+  const int lo = ab_first_key(p, qi), n = qi + 1 - lo;
+  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
+  j_lo = lo + min(n, sp * per);
+  j_hi = min(lo + n, j_lo + per);
+}
+
 // prefill: grid (ceil(S / 4), H, B), one wave per query
 template <typename CT, int VREG>
 __global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
@@ -161,7 +176,7 @@ __global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
   __builtin_amdgcn_wave_barrier();
   const int qi = min(*p.slot + s, p.T - 1);
   float m_run, l_run, acc[VREG];
-  ab_wave<CT, VREG>(p, qs, b, h, qi, 0, qi + 1, true, m_run, l_run, acc);
+  ab_wave<CT, VREG>(p, qs, b, h, qi, ab_first_key(p, qi), qi + 1, true, m_run, l_run, acc);
   float* o = p.out + ((size_t)b * p.S + s) * (p.H * p.vdim) + (size_t)h * p.vdim;
   const float inv = 1.f / l_run;
 #pragma unroll
@@ -181,9 +196,8 @@ __global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
   for (int d = lane; d < p.dim; d += 64) qs[d] = q[d];
   __syncthreads();
   const int qi = min(*p.slot, p.T - 1);
-  const int n = qi + 1;
-  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
-  const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
+  int j_lo, j_hi;
+  ab_split_range(p, qi, sp, j_lo, j_hi);
   float m_run, l_run, acc[VREG];
   ab_wave<CT, VREG>(p, qs, b, h, qi, j_lo, j_hi, sp == 0, m_run, l_run, acc);
   float* w = p.ws + (((size_t)b * p.H + h) * p.splits + sp) * (p.vdim + 2);
@@ -213,12 +227,12 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
 #pragma unroll
   for (int i = 0; i < dim / 64; ++i) qv[i] = q[lane + 64 * i];
   const int qi = min(*p.slot, p.T - 1);
-  const int n = qi + 1;
-  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
-  const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
+  int j_lo, j_hi;
+  ab_split_range(p, qi, sp, j_lo, j_hi);
   const bf16_t* kbase = reinterpret_cast<const bf16_t*>(p.kc) + ((size_t)b * p.G + g) * p.T * dim;
   const bf16_t* vbase = reinterpret_cast<const bf16_t*>(p.vc) + ((size_t)b * p.G + g) * p.T * vdim;
   const bool sunk = p.sink && sp == 0;
+  const float hs = p.head_scale ? p.head_scale[h] : 1.f;
   float m_run = sunk ? p.sink[h] : -INFINITY, l_run = sunk ? 1.f : 0.f, acc[VREG];
 #pragma unroll
   for (int i = 0; i < VREG; ++i) acc[i] = 0.f;
@@ -253,7 +267,7 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
         d1 = fmaf(qs[8 * u + i + 1], f[i + 1], d1);
       }
     }
-    float sc = (d0 + d1) * p.scale;
+    float sc = (d0 + d1) * p.scale * hs;
     if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
     sc += bl;
     if (j >= j_hi) sc = -INFINITY;
@@ -308,14 +322,14 @@ __global__ void __launch_bounds__(64) attn_latent_decode_kernel(AttnBias p) {
     for (int i = 0; i < 8; ++i) qv[q][i] = on ? qv[q][i] : 0.f;
   }
   const int qi = min(*p.slot, p.T - 1);
-  const int n = qi + 1;
-  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
-  const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
+  int j_lo, j_hi;
+  ab_split_range(p, qi, sp, j_lo, j_hi);
   const bf16_t* base = reinterpret_cast<const bf16_t*>(p.kc) + (size_t)b * p.T * rank + c0;
   const bool sunk = p.sink && sp == 0;
-  float m_run[HQ], l_run[HQ], acc[HQ][8];
+  float m_run[HQ], l_run[HQ], acc[HQ][8], hs[HQ];
 #pragma unroll
   for (int q = 0; q < HQ; ++q) {
+    hs[q] = p.head_scale ? p.head_scale[h0 + q] : 1.f;
     m_run[q] = sunk ? p.sink[h0 + q] : -INFINITY;
     l_run[q] = sunk ? 1.f : 0.f;
 #pragma unroll
@@ -342,7 +356,7 @@ __global__ void __launch_bounds__(64) attn_latent_decode_kernel(AttnBias p) {
           d1 = fmaf(qv[q][i + 1], f[i + 1], d1);
         }
         const float rt = row16_sum(d0 + d1);
-        const float dot = (al_lane(rt, 0) + al_lane(rt, 16) + al_lane(rt, 32) + al_lane(rt, 48)) * p.scale;
+        const float dot = (al_lane(rt, 0) + al_lane(rt, 16) + al_lane(rt, 32) + al_lane(rt, 48)) * p.scale * hs[q];
         sc[q][u] = j0 + u < j_hi ? dot : -INFINITY;
         cmax[q] = fmaxf(cmax[q], sc[q][u]);
       }
@@ -483,6 +497,10 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
   float m_run = p.sink ? p.sink[h] : -INFINITY, l_run = p.sink && hi == 0 ? 1.f : 0.f;
   const int q_last = min(q0 + AM_Q - 1, slot + p.S - 1);
   const float inv_cap = p.softcap > 0.f ? 1.f / p.softcap : 0.f;
+  const float hs = p.head_scale ? p.head_scale[h] : 1.f;
+  // block-local mask: this query's first key, the last query's (the largest of the wave), and the tile the walk starts at
+  const int lo_q = ab_first_key(p, qi), lo_last = ab_first_key(p, q_last);
+  const int j_begin = ab_first_key(p, q0) / AM_K * AM_K;
   // the next tile's key and value fragments are loaded while the current tile is computed (one wave per SIMD at small
   // batch: nothing else hides the loads)
   u32x4 kn[DK], vn[2][VT];
@@ -496,8 +514,8 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
       for (int v = 0; v < VT; ++v)
         vn[c][v] = *reinterpret_cast<const u32x4*>(vbase + (size_t)(32 * v + ql) * Tp + min(j0, Tp - AM_K) + 16 * c + 8 * hi);
   };
-  fetch(0);
-  for (int j0 = 0; j0 <= q_last; j0 += AM_K) {
+  fetch(j_begin);
+  for (int j0 = j_begin; j0 <= q_last; j0 += AM_K) {
     u32x4 kc_[DK], vc_[2][VT];
 #pragma unroll
     for (int kk = 0; kk < DK; ++kk) kc_[kk] = kn[kk];
@@ -518,26 +536,28 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
     const int dbase = q0 - j0 - (AM_K - 1);
     const bool far = p.bias && dbase >= p.nbias - 1;
     if (p.bias) bl = p.bias[(size_t)min(max(dbase + lane, 0), p.nbias - 1) * p.H + h];
-    const bool diag = j0 + AM_K - 1 > q0;  // some (query, key) of the tile is masked
+    const bool diag = j0 + AM_K - 1 > q0 || j0 < lo_last;  // some (query, key) of the tile is masked
     float tmax = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kl = 16 * (r >> 3) + 8 * hi + (r & 7);  // key of accumulator r within the tile
-      float sc = sacc[r] * p.scale;
+      float sc = sacc[r] * p.scale * hs;
       if (p.softcap > 0.f) sc = p.softcap * am_tanh(sc * inv_cap);
       if (p.bias) sc += far ? bl : __shfl(bl, ql - kl + (AM_K - 1), 64);
-      if (diag && j0 + kl > qi) sc = -INFINITY;
+      if (diag && (j0 + kl > qi || j0 + kl < lo_q)) sc = -INFINITY;
       sacc[r] = sc;
       tmax = fmaxf(tmax, sc);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m_run, tmax);
-    const float corr = __expf(m_run - m_new);
+    // (a query without a sink may have no visible key in a tile it shares with its neighbours' earlier blocks)
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __expf(m_run - m_use);
     m_run = m_new;
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sacc[r] = __expf(sacc[r] - m_new);
+      sacc[r] = __expf(sacc[r] - m_use);
       psum += sacc[r];
     }
     l_run = l_run * corr + psum;  // (this half-wave's keys; the halves are added at the end)
@@ -626,6 +646,7 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
   if (p.B < 0 || p.S < 1 || p.H < 1 || p.G < 1 || p.H % p.G || p.T < 1) return -1;
   if (p.dim < 1 || p.dim > AB_MAX_DIM || p.vdim < 1 || p.vdim > 64 * AB_MAX_VREG) return -2;
   if (p.bias && p.nbias < 1) return -3;
+  if (p.chunk < 0) return -7;
   if (p.B == 0) return 0;
   if (p.H > 65535 || p.B > 65535) return -4;
   if (p.S == 1) {

@@ -76,15 +76,16 @@ void embed_rows(Tensor ids, Tensor table, int64_t col0, Tensor out, double scale
 
 void linear_rows(Tensor a, OptT a_idx, Tensor w, Tensor out, OptT dst_idx, OptT offs, OptT row_expert, int64_t R,
                  int64_t act, double act_limit, double act_alpha, OptT a_scale, OptT a_norm_w, double a_norm_eps,
-                 int64_t even_rows) {
+                 int64_t even_rows, bool add_out) {
   jla::RowLinear p{};
   p.even_rows = even_rows;
+  p.add_out = add_out;
   p.wbf16 = wtype(w, "w");
   check(w.dim() == 2 || w.dim() == 3, "linear_rows: w is [Nw, K] or [E, Nw, K]");
   p.E = w.dim() == 3 ? w.size(0) : 1;
   const int64_t Nw = w.size(-2);
   p.K = w.size(-1);
-  check(act >= jla::HY_ACT_NONE && act <= jla::HY_ACT_CLAMP_GLU, "linear_rows: unknown activation");
+  check(act >= jla::HY_ACT_NONE && act <= jla::HY_ACT_SOFTCAP, "linear_rows: unknown activation");
   const bool gated = jla::hy_act_gated(act);
   check(!gated || Nw % 2 == 0, "linear_rows: a gated activation needs gate and up rows");
   p.N = gated ? Nw / 2 : Nw;
@@ -265,7 +266,7 @@ int64_t attn_prefill_ws_bytes(int64_t B, int64_t S, int64_t G, int64_t dim, int6
 }
 
 void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double softcap, OptT bias, Tensor out,
-               int64_t t_cap, OptT ws, int64_t splits, OptT vt_ws, OptT sink) {
+               int64_t t_cap, OptT ws, int64_t splits, OptT vt_ws, OptT sink, int64_t chunk, OptT head_scale) {
   jla::AttnBias p{};
   check(q.dim() == 4, "attn_bias: q is [B, S, H, dim]");
   p.B = q.size(0); p.S = q.size(1); p.H = q.size(2); p.dim = q.size(3);
@@ -289,6 +290,12 @@ void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double
   if (sink.has_value()) {
     check(sink->numel() == p.H, "attn_bias: sink is [H]");
     p.sink = f32(*sink, "sink");
+  }
+  check(chunk >= 0 && chunk <= INT32_MAX, "attn_bias: chunk");
+  p.chunk = chunk;
+  if (head_scale.has_value()) {
+    check(head_scale->numel() == p.H, "attn_bias: head_scale is [H]");
+    p.head_scale = f32(*head_scale, "head_scale");
   }
   check(out.numel() == (int64_t)p.B * p.S * p.H * p.vdim, "attn_bias: out shape");
   p.out = f32w(out, "out");
@@ -367,14 +374,154 @@ void delta_scan(Tensor qn, Tensor kn, Tensor v, Tensor beta, Tensor decay, Tenso
   rc(jla::hy_delta_scan(p, stream()), "delta_scan");
 }
 
-void gated_rmsnorm(Tensor o, Tensor gate, Tensor w, double eps, Tensor out, int64_t H, int64_t vdim) {
-  const int64_t M = o.numel() / (H * vdim);
-  check(o.numel() == M * H * vdim && out.numel() == o.numel() && w.numel() == vdim, "gated_rmsnorm shapes");
-  int ldg = 0;
+// a 2-d float32 view with unit inner stride whose rows hold at least `cols` numbers
+float* slice2d(const Tensor& t, const char* name, int64_t rows, int64_t cols, int* ld) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.dim() == 2 && t.stride(1) == 1 &&
+                  t.size(0) == rows && t.size(1) == cols && (rows <= 1 || t.stride(0) >= cols),
+              "jax_llama_amd._C_hybrid: ", name, " must be a float32 [", rows, ", ", cols,
+              "] GPU view with unit inner stride");
+  *ld = rows > 1 ? (int)t.stride(0) : (int)cols;
+  return reinterpret_cast<float*>(t.data_ptr());
+}
+
+// a [M, H, n] float32 view whose heads are adjacent (stride(1) == n, unit inner stride): rows may be strided
+const float* heads3d(const Tensor& t, const char* name, int64_t M, int64_t H, int64_t n, int* ld) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.dim() == 3 && t.size(0) == M && t.size(1) == H &&
+                  t.size(2) == n && t.stride(2) == 1 && (H == 1 || t.stride(1) == n) && (M <= 1 || t.stride(0) >= H * n),
+              "jax_llama_amd._C_hybrid: ", name, " must be a float32 [", M, ", ", H, ", ", n,
+              "] GPU view with adjacent heads");
+  *ld = M > 1 ? (int)t.stride(0) : (int)(H * n);
+  return reinterpret_cast<const float*>(t.data_ptr());
+}
+
+const double* f64(const Tensor& t, const char* name) {
+  gpu(t, name);
+  TORCH_CHECK(t.scalar_type() == torch::kFloat64, "jax_llama_amd._C_hybrid: ", name, " must be float64");
+  return reinterpret_cast<const double*>(t.data_ptr());
+}
+
+void gated_rmsnorm(Tensor o, Tensor gate, Tensor w, double eps, Tensor out, int64_t H, int64_t vdim, int64_t gate_act,
+                   OptT denom_floor, double gain) {
+  jla::GatedNorm p{};
+  const int64_t ov = denom_floor.has_value() ? vdim + 1 : vdim;
+  const int64_t M = o.numel() / (H * ov);
+  check(o.numel() == M * H * ov && (w.numel() == vdim || w.numel() == H * vdim), "gated_rmsnorm shapes");
   check(gate.dim() == 2 && gate.size(0) == M, "gated_rmsnorm: gate rows");
-  const float* g = rows2d(gate, "gate", H * vdim, &ldg);
-  rc(jla::hy_gated_rmsnorm(f32(o, "o"), g, ldg, f32(w, "w"), (float)eps, f32w(out, "out"), M, H, vdim, stream()),
-     "gated_rmsnorm");
+  p.o = f32(o, "o");
+  p.gate = rows2d(gate, "gate", H * vdim, &p.ldg);
+  p.w = f32(w, "w");
+  p.w_heads = w.numel() != vdim || H == 1;
+  p.eps = eps;
+  p.out = slice2d(out, "out", M, H * vdim, &p.ldo);
+  p.M = M; p.H = H; p.vdim = vdim;
+  p.gate_act = gate_act;
+  if (denom_floor.has_value()) {
+    check(denom_floor->numel() == M * H, "gated_rmsnorm: denom_floor is [M, H]");
+    p.denom_floor = f32(*denom_floor, "denom_floor");
+  }
+  p.gain = gain;
+  rc(jla::hy_gated_rmsnorm(p, stream()), "gated_rmsnorm");
+}
+
+void rope_prep(Tensor proj, OptT bias, Tensor positions, Tensor slot, int64_t B, int64_t S, int64_t H, int64_t G,
+               int64_t dim, int64_t vdim, Tensor kc, Tensor vc, Tensor q, Tensor qk_freq, OptT v_freq) {
+  jla::RopePrep p{};
+  const int64_t cols = (H + G) * dim + G * vdim;
+  check(proj.dim() == 2 && proj.size(0) == B * S, "rope_prep: proj rows");
+  p.proj = rows2d(proj, "proj", cols, &p.ld);
+  if (bias.has_value()) {
+    check(bias->numel() == cols, "rope_prep: one bias per projection column");
+    p.bias = f32(*bias, "bias");
+  }
+  p.positions = i32(positions, "positions", B * S);
+  p.slot = i32(slot, "slot", 1);
+  p.B = B; p.S = S; p.H = H; p.G = G; p.dim = dim; p.vdim = vdim;
+  p.cbf16 = wtype(kc, "k cache");
+  check(wtype(vc, "v cache") == p.cbf16, "rope_prep: cache dtypes differ");
+  check(kc.dim() == 4 && kc.size(0) == B && kc.size(1) == G && kc.size(3) == dim, "rope_prep: k cache shape");
+  p.T = kc.size(2);
+  check(vc.dim() == 4 && vc.size(0) == B && vc.size(1) == G && vc.size(2) == p.T && vc.size(3) == vdim,
+        "rope_prep: v cache shape");
+  p.kc = kc.data_ptr();
+  p.vc = vc.data_ptr();
+  check(q.numel() == B * S * H * dim, "rope_prep: q shape");
+  p.q = f32w(q, "q");
+  p.qk_half = qk_freq.numel();
+  check(2 * p.qk_half <= dim, "rope_prep: more rotated numbers than a head holds");
+  p.qk_freq = p.qk_half ? f64(qk_freq, "qk_freq") : nullptr;
+  if (v_freq.has_value() && v_freq->numel() > 0) {
+    p.v_half = v_freq->numel();
+    check(2 * p.v_half <= vdim, "rope_prep: more rotated numbers than a value head holds");
+    p.v_freq = f64(*v_freq, "v_freq");
+  }
+  rc(jla::hy_rope_prep(p, stream()), "rope_prep");
+}
+
+void rotate_heads(Tensor a, Tensor positions, OptT freq, int64_t H, double sign, double gain, Tensor out) {
+  check(a.dim() == 2 && a.size(1) % H == 0, "rotate_heads: a is [M, H * n]");
+  const int64_t M = a.size(0), n = a.size(1) / H;
+  int lda = 0, ldo = 0;
+  const float* ap = slice2d(a, "a", M, H * n, &lda);
+  float* op = slice2d(out, "out", M, H * n, &ldo);
+  const int half = freq.has_value() ? (int)freq->numel() : 0;
+  check(2 * half <= n, "rotate_heads: more rotated numbers than a head holds");
+  rc(jla::hy_rotate_heads(ap, lda, i32(positions, "positions", M), half ? f64(*freq, "freq") : nullptr, half, M, H, n,
+                          (float)sign, (float)gain, op, ldo, stream()),
+     "rotate_heads");
+}
+
+void token_shift(Tensor h, Tensor prev, Tensor mu, Tensor out, int64_t B, int64_t S) {
+  check(mu.dim() == 2, "token_shift: mu is [n, D]");
+  const int64_t n = mu.size(0), D = mu.size(1);
+  check(h.numel() == B * S * D && prev.numel() == B * D && out.numel() == n * B * S * D, "token_shift shapes");
+  rc(jla::hy_token_shift(f32(h, "h"), f32w(prev, "prev"), f32(mu, "mu"), n, f32w(out, "out"), B, S, D, stream()),
+     "token_shift");
+}
+
+void mlstm_prep(Tensor proj, int64_t col_i, int64_t col_f, Tensor gate_bias, double cap, Tensor mstate, Tensor out,
+                int64_t B, int64_t S, int64_t H) {
+  jla::MlstmPrep p{};
+  check(proj.dim() == 2 && proj.size(0) == B * S, "mlstm_prep: proj rows");
+  p.proj = rows2d(proj, "proj", proj.size(1), &p.ld);
+  check(col_i >= 0 && col_f >= 0 && col_i + H <= proj.size(1) && col_f + H <= proj.size(1), "mlstm_prep: gate columns");
+  p.col_i = col_i; p.col_f = col_f;
+  check(gate_bias.numel() == 2 * H && mstate.numel() == B * H && out.numel() == 3 * B * S * H, "mlstm_prep shapes");
+  p.gate_bias = f32(gate_bias, "gate_bias");
+  p.cap = cap;
+  p.mstate = f32w(mstate, "mstate");
+  float* o = f32w(out, "out");
+  p.keep = o; p.write = o + B * S * H; p.floor = o + 2 * B * S * H;
+  p.B = B; p.S = S; p.H = H;
+  rc(jla::hy_mlstm_prep(p, stream()), "mlstm_prep");
+}
+
+void lin_scan(int64_t mode, Tensor q, Tensor k, Tensor v, Tensor decay, OptT write, OptT w0, OptT u, Tensor state,
+              Tensor o, int64_t B, int64_t S, double q_scale) {
+  jla::LinScan p{};
+  check(mode == 0 || mode == 1, "lin_scan: mode");
+  check(q.dim() == 3 && v.dim() == 3, "lin_scan: q, k are [M, H, dim], v is [M, H, vdim]");
+  const int64_t M = B * S, H = q.size(1), dim = q.size(2), vdim = v.size(2);
+  const int64_t cols = mode == 0 ? vdim + 1 : vdim;
+  p.mode = mode;
+  p.q = heads3d(q, "q", M, H, dim, &p.ldq);
+  p.k = heads3d(k, "k", M, H, dim, &p.ldk);
+  p.v = heads3d(v, "v", M, H, vdim, &p.ldv);
+  if (mode == 0) {
+    check(decay.numel() == M * H && write.has_value() && write->numel() == M * H, "lin_scan: keep, write are [M, H]");
+    p.decay = f32(decay, "keep");
+    p.write = f32(*write, "write");
+  } else {
+    p.decay = heads3d(decay, "decay", M, H, dim, &p.ldd);
+    check(w0.has_value() && u.has_value() && w0->numel() == H * dim && u->numel() == H * dim, "lin_scan: w0, u are [H, dim]");
+    p.w0 = f32(*w0, "w0");
+    p.u = f32(*u, "u");
+  }
+  check(state.numel() == B * H * dim * cols && o.numel() == M * H * cols, "lin_scan: state / output shapes");
+  p.state = f32w(state, "state");
+  p.o = f32w(o, "o");
+  p.B = B; p.S = S; p.H = H; p.dim = dim; p.vdim = vdim;
+  p.q_scale = q_scale;
+  rc(jla::hy_lin_scan(p, stream()), "lin_scan");
 }
 
 }  // namespace
@@ -384,7 +531,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_rows", &embed_rows);
   m.def("linear_rows", &linear_rows, py::arg("a"), py::arg("a_idx"), py::arg("w"), py::arg("out"), py::arg("dst_idx"),
         py::arg("offs"), py::arg("row_expert"), py::arg("R"), py::arg("act"), py::arg("act_limit"), py::arg("act_alpha"),
-        py::arg("a_scale"), py::arg("a_norm_w"), py::arg("a_norm_eps"), py::arg("even_rows") = 0);
+        py::arg("a_scale"), py::arg("a_norm_w"), py::arg("a_norm_eps"), py::arg("even_rows") = 0,
+        py::arg("add_out") = false);
   m.def("route_table", &route_table);
   m.def("route_topk", &route_topk);
   m.def("dense_is_gemv", &dense_is_gemv);
@@ -398,10 +546,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("cast_bf16", &cast_bf16);
   m.def("attn_prep", &attn_prep);
   m.def("attn_decode_splits", &attn_decode_splits);
-  m.def("attn_bias", &attn_bias);
+  m.def("attn_bias", &attn_bias, py::arg("q"), py::arg("kc"), py::arg("vc"), py::arg("slot"), py::arg("scale"),
+        py::arg("softcap"), py::arg("bias"), py::arg("out"), py::arg("t_cap"), py::arg("ws"), py::arg("splits"),
+        py::arg("vt_ws"), py::arg("sink"), py::arg("chunk") = 0, py::arg("head_scale") = py::none());
   m.def("attn_prefill_ws_bytes", &attn_prefill_ws_bytes);
   m.def("delta_prep", &delta_prep);
   m.def("conv_state_update", &conv_state_update);
   m.def("delta_scan", &delta_scan);
-  m.def("gated_rmsnorm", &gated_rmsnorm);
+  m.def("gated_rmsnorm", &gated_rmsnorm, py::arg("o"), py::arg("gate"), py::arg("w"), py::arg("eps"), py::arg("out"),
+        py::arg("H"), py::arg("vdim"), py::arg("gate_act") = 0, py::arg("denom_floor") = py::none(),
+        py::arg("gain") = 1.0);
+  m.attr("ACT_SOFTCAP") = (int)jla::HY_ACT_SOFTCAP;
+  m.def("rope_prep", &rope_prep);
+  m.def("rotate_heads", &rotate_heads);
+  m.def("token_shift", &token_shift);
+  m.def("mlstm_prep", &mlstm_prep);
+  m.def("lin_scan", &lin_scan);
 }

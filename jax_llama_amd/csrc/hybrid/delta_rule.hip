@@ -13,7 +13,8 @@
 //   hy_delta_scan        : the recurrence, token by token. A thread owns 16 key rows of one value column in registers;
 //                          the lanes sharing a column (dim / 16 of them, adjacent) combine their partial S^T k and
 //                          S^T q by lane exchange. k, q, v, g, beta of the next tokens are staged through LDS.
-//   hy_gated_rmsnorm     : o / rms(o) * w * silu(gate) per head.
+//   hy_gated_rmsnorm     : o / rms(o) * w * act(gate) per head (silu or sigmoid; the gain per column or per head and
+//                          column; optionally o first divided by its own normaliser column).
 #include "hy_util.h"
 #include "hybrid.h"
 
@@ -250,27 +251,36 @@ int hy_delta_scan(const DeltaScan& p, hipStream_t s) {
 }
 
 // grid (M, ceil(H / 4)), one wave per (token, head)
-__global__ void __launch_bounds__(256) gated_rmsnorm_kernel(const float* o, const float* gate, int ldg, const float* w,
-                                                            float eps, float* out, int M, int H, int vdim) {
+__global__ void __launch_bounds__(256) gated_rmsnorm_kernel(GatedNorm p) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = blockIdx.x, h = blockIdx.y * 4 + wave;
-  if (h >= H) return;
-  const float* x = o + ((size_t)m * H + h) * vdim;
+  if (h >= p.H) return;
+  const int vdim = p.vdim, ov = p.denom_floor ? vdim + 1 : vdim;
+  const float* x = p.o + ((size_t)m * p.H + h) * ov;
+  float pre = 1.f;  // the read-out's own normaliser, applied before the statistic
+  if (p.denom_floor) pre = 1.f / (fmaxf(fabsf(x[vdim]), p.denom_floor[(size_t)m * p.H + h]) + 1e-6f);
   float ss = 0.f;
-  for (int d = lane; d < vdim; d += 64) ss = fmaf(x[d], x[d], ss);
+  for (int d = lane; d < vdim; d += 64) {
+    const float v = x[d] * pre;
+    ss = fmaf(v, v, ss);
+  }
   ss = wave_sum(ss);
-  const float sc = 1.f / sqrtf(ss / (float)vdim + eps);
-  const float* gr = gate + (size_t)m * ldg + (size_t)h * vdim;
-  float* dst = out + ((size_t)m * H + h) * vdim;
-  for (int d = lane; d < vdim; d += 64) dst[d] = x[d] * sc * w[d] * hy_silu(gr[d]);
+  const float sc = 1.f / sqrtf(ss / (float)vdim + p.eps);
+  const float* gr = p.gate + (size_t)m * p.ldg + (size_t)h * vdim;
+  const float* w = p.w + (p.w_heads ? (size_t)h * vdim : 0);
+  float* dst = p.out + (size_t)m * p.ldo + (size_t)h * vdim;
+  for (int d = lane; d < vdim; d += 64) {
+    const float g = p.gate_act == 1 ? hy_sigmoid(gr[d]) : hy_silu(gr[d]);
+    dst[d] = (x[d] * pre) * sc * w[d] * g * p.gain;
+  }
 }
 
-int hy_gated_rmsnorm(const float* o, const float* gate, int ldg, const float* w, float eps, float* out, int M, int H,
-                     int vdim, hipStream_t s) {
-  if (M < 0 || H < 1 || vdim < 1 || ldg < H * vdim) return -1;
-  if (M == 0) return 0;
-  if ((H + 3) / 4 > 65535) return -2;
-  gated_rmsnorm_kernel<<<dim3(M, (H + 3) / 4), 256, 0, s>>>(o, gate, ldg, w, eps, out, M, H, vdim);
+int hy_gated_rmsnorm(const GatedNorm& p, hipStream_t s) {
+  if (p.M < 0 || p.H < 1 || p.vdim < 1 || p.ldg < p.H * p.vdim || p.ldo < p.H * p.vdim) return -1;
+  if (p.gate_act != 0 && p.gate_act != 1) return -3;
+  if (p.M == 0) return 0;
+  if ((p.H + 3) / 4 > 65535) return -2;
+  gated_rmsnorm_kernel<<<dim3(p.M, (p.H + 3) / 4), 256, 0, s>>>(p);
   JLA_CHECK_LAUNCH();
   return 0;
 }

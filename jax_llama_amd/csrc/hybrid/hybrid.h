@@ -22,6 +22,7 @@ enum RowAct {
   HY_ACT_RELU2 = 1,       // out = max(y, 0)^2
   HY_ACT_SWIGLU = 2,      // out = silu(g) * u
   HY_ACT_CLAMP_GLU = 3,   // g = min(g, limit), u = clamp(u, -limit, limit): out = g * sigmoid(alpha g) * (u + 1)
+  HY_ACT_SOFTCAP = 4,     // out = limit * tanh(y / limit)   (limit = 1: tanh)
 };
 
 struct RowLinear {
@@ -49,6 +50,7 @@ struct RowLinear {
   int act;               // RowAct; the gated forms read W as [2N, K]
   float act_limit;       // HY_ACT_CLAMP_GLU
   float act_alpha;
+  int add_out;           // out += act(...) instead of out = (fp32 outputs): a residual add in the epilogue
 };
 inline bool hy_act_gated(int act) { return act == HY_ACT_SWIGLU || act == HY_ACT_CLAMP_GLU; }
 // R <= HY_GEMV_MAX_R and (offs == nullptr or row_expert != nullptr): one wave per output column (weights streamed once
@@ -139,6 +141,8 @@ struct AttnBias {
   float* ws;   // decode split partials: B * H * splits * (vdim + 2) floats
   int splits;
   void* vt_ws;  // prefill: hy_attn_prefill_ws_bytes(...) bytes for the transposed values (nullptr: the plain kernel)
+  int chunk;    // > 0: query at slot i sees only keys j <= i with floor(j / chunk) == floor(i / chunk)
+  const float* head_scale;  // optional [H]: head h's scores are (q . k * scale) * head_scale[h]
 };
 int hy_attn_bias(const AttnBias& p, hipStream_t s);
 long long hy_attn_prefill_ws_bytes(int B, int S, int G, int dim, int vdim, int T, int cbf16);
@@ -173,8 +177,91 @@ struct DeltaScan {
 };
 int hy_delta_scan(const DeltaScan& p, hipStream_t s);
 
-// out[m, h * vdim + j] = o[m, h, j] / sqrt(mean_j(o^2) + eps) * w[j] * silu(gate[m * ldg + h * vdim + j])
-int hy_gated_rmsnorm(const float* o, const float* gate, int ldg, const float* w, float eps, float* out, int M, int H,
-                     int vdim, hipStream_t s);
+// out[m * ldo + h * vdim + j] = x[m, h, j] / sqrt(mean_j(x^2) + eps) * w[w_heads ? h * vdim + j : j] *
+// act(gate[m * ldg + h * vdim + j]) * gain, act = silu (gate_act 0) or sigmoid (1). x = o, or with denom_floor [M, H]:
+// o is [M, H, vdim + 1] and x[m, h, j] = o[m, h, j] / (max(|o[m, h, vdim]|, denom_floor[m, h]) + 1e-6).
+struct GatedNorm {
+  const float* o;
+  const float* gate;
+  int ldg;
+  const float* w;
+  int w_heads;
+  float eps;
+  float* out;
+  int ldo;
+  int M, H, vdim;
+  int gate_act;
+  const float* denom_floor;
+  float gain;
+};
+int hy_gated_rmsnorm(const GatedNorm& p, hipStream_t s);
+
+// Rotary positions for a fused q | k | v projection (+ bias per column): q and k heads rotated on their first 2 qk_half
+// numbers (number i with i + qk_half, angle position * qk_freq[i]), v heads on their first 2 v_half numbers when v_freq
+// is given; q to a dense buffer, k / v into the caches at slot + s. Angles are formed in 64-bit.
+struct RopePrep {
+  const float* proj;  // [M, ld]: q heads, k heads, v heads
+  int ld;
+  const float* bias;  // optional [H dim + G dim + G vdim]
+  const int32_t* positions;  // [M]
+  const int32_t* slot;
+  int B, S, H, G, dim, vdim, T;
+  void* kc;  // [B, G, T, dim]
+  void* vc;  // [B, G, T, vdim]
+  int cbf16;
+  float* q;  // [M, H, dim]
+  const double* qk_freq;
+  int qk_half;
+  const double* v_freq;  // optional
+  int v_half;
+};
+int hy_rope_prep(const RopePrep& p, hipStream_t s);
+
+// out[m * ldo + h * n + d] = gain * turn(a[m * lda + h * n + .], sign * positions[m])[d]: the first 2 half numbers of
+// every head rotated (freq == nullptr: none, a scaled copy)
+int hy_rotate_heads(const float* a, int lda, const int32_t* positions, const double* freq, int half, int M, int H, int n,
+                    float sign, float gain, float* out, int ldo, hipStream_t s);
+
+// out[i][m][:] = h[m] + (h[m - 1] - h[m]) * mu[i] for i < n; the row before a sequence's first is prev[b] (then set to
+// the sequence's last row)
+int hy_token_shift(const float* h, float* prev, const float* mu, int n, float* out, int B, int S, int D, hipStream_t s);
+
+struct MlstmPrep {
+  const float* proj;  // [M, ld]: input-gate pre-activations at columns [col_i, col_i + H), forget-gate at [col_f, col_f + H)
+  int ld, col_i, col_f;
+  const float* gate_bias;  // [2 H]
+  float cap;
+  float* mstate;  // [B, H] running maximum, read and advanced
+  float* keep;    // [M, H] exp(f + m' - m)
+  float* write;   // [M, H] exp(a - m)
+  float* floor;   // [M, H] exp(-m)
+  int B, S, H;
+};
+int hy_mlstm_prep(const MlstmPrep& p, hipStream_t s);
+
+// Linear recurrences over a matrix state [B, H, dim, cols] (fp32), token by token.
+//   mode 0 (scalar gates, read after the write; cols = vdim + 1, the last column's value is 1):
+//       S <- keep S + write k [v, 1]^T;   o = S^T (q_scale q)
+//   mode 1 (a decay per key channel, bonus u for the current token, read before the write; cols = vdim):
+//       d = exp(-exp(decay + w0));   o = (S + diag(u) k v^T)^T q;   S <- diag(d) S + k v^T
+struct LinScan {
+  int mode;
+  const float* q;  // token m, head h at q + m * ldq + h * dim
+  int ldq;
+  const float* k;
+  int ldk;
+  const float* v;  // token m, head h at v + m * ldv + h * vdim
+  int ldv;
+  const float* decay;  // mode 0: keep [M, H]; mode 1: pre-activations, token m, head h at decay + m * ldd + h * dim
+  int ldd;
+  const float* write;  // mode 0: [M, H]
+  const float* w0;     // mode 1: [H, dim]
+  const float* u;      // mode 1: [H, dim]
+  float* state;
+  float* o;  // [M, H, cols]
+  int B, S, H, dim, vdim;
+  float q_scale;
+};
+int hy_lin_scan(const LinScan& p, hipStream_t s);
 
 }  // namespace jla

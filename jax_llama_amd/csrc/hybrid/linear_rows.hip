@@ -105,10 +105,14 @@ JLA_DEV float lr_act(const RowLinear& p, float g, float u) {
       const float gc = fminf(g, p.act_limit), uc = fminf(fmaxf(u, -p.act_limit), p.act_limit);
       return gc * hy_sigmoid(p.act_alpha * gc) * (uc + 1.f);
     }
+    case HY_ACT_SOFTCAP:
+      return p.act_limit * tanhf(g / p.act_limit);
     default:
       return g;
   }
 }
+JLA_DEV float lr_in(const float* p) { return *p; }
+JLA_DEV float lr_in(const bf16_t* p) { return bf2f(*p); }
 
 // WT: weight / tile type; AT: activation type in memory (fp32, or a bf16 copy); OT: output type; TMM: 32-row tiles per
 // wave along M (workgroup tile 64 TMM x 64: the 128-row form halves the weight traffic per output row).
@@ -197,7 +201,9 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
       const int row = r0 + wm * 32 * TMM + 32 * t + (r & 3) + 8 * (r >> 2) + 4 * hi;
       if (row < rend) {
         const int drow = p.dst_idx ? p.dst_idx[row] : row;
-        lr_out(out + (size_t)drow * p.ldo + col, lr_act(p, acc[t][r], SWIGLU ? acc2[t][r] : 0.f));
+        OT* dst = out + (size_t)drow * p.ldo + col;
+        const float val = lr_act(p, acc[t][r], SWIGLU ? acc2[t][r] : 0.f);
+        lr_out(dst, p.add_out ? lr_in(dst) + val : val);
       }
     }
 }
@@ -313,8 +319,11 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
       for (int c = 0; c < LR_CPW; ++c) {
         const float g = wave_sum(acc[r][c]);
         const float u = SWIGLU ? wave_sum(acc2[r][c]) : 0.f;
-        if (lane == 0 && n0 + c < p.N)
-          reinterpret_cast<float*>(p.out)[(size_t)drow * p.ldo + n0 + c] = lr_act(p, g, u);
+        if (lane == 0 && n0 + c < p.N) {
+          float* dst = reinterpret_cast<float*>(p.out) + (size_t)drow * p.ldo + n0 + c;
+          const float val = lr_act(p, g, u);
+          *dst = p.add_out ? *dst + val : val;
+        }
       }
     }
   }
@@ -339,7 +348,9 @@ bool hy_linear_rows_is_gemv(const RowLinear& p) {
 
 int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   if (p.R < 0 || p.N <= 0 || p.K <= 0 || p.lda < p.K || p.ldo < p.N || p.E < 1) return -1;
-  if (p.act < HY_ACT_NONE || p.act > HY_ACT_CLAMP_GLU) return -8;
+  if (p.act < HY_ACT_NONE || p.act > HY_ACT_SOFTCAP) return -8;
+  if (p.act == HY_ACT_SOFTCAP && !(p.act_limit > 0.f)) return -8;
+  if (p.add_out && p.out_bf16) return -11;
   if (p.a_scale && p.a_bf16) return -9;  // (a bf16 copy cannot be scaled before its rounding)
   const int gated = hy_act_gated(p.act);
   if (p.R == 0) return 0;
