@@ -559,6 +559,9 @@ def test_longer_prompts_at_the_kernel_shapes(dtype):
     model = BesulixForCausalLM(BesulixConfig.from_dict(cfg), device="cuda", dtype=dtype, _do_init=False).load_state_dict(sd)
     got = run_portions(model, t, [261, 3, 2, 190, 64, 37] + [1] * 43)
     e = np.array([err(got[i], ref[i]) for i in range(600)])
-    assert e.max() < (2e-4 if dtype == F32 else 4e-2), (int(np.argmax(e)), e.max())
+    # (bf16: six layers of rounded operands; the largest of 600 rows sits a few times above the typical one, while a
+    # wrong mask, state or position puts a row at order 1)
+    assert e.max() < (2e-4 if dtype == F32 else 8e-2), (int(np.argmax(e)), e.max())
+    assert e.mean() < (5e-5 if dtype == F32 else 1.5e-2), e.mean()
     whole = run_portions(model, t, [600])
     assert err(whole, got) < (2e-5 if dtype == F32 else 2e-2)
