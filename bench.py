@@ -81,12 +81,18 @@ def main():
     ap.add_argument("--latent-compare", action="store_true", help="the same comparison for the latent-attention family: "
                     "Zasevik beside Zavevik (the closest family) and LLaMA (--hybrid-compare --hybrid-families zasevik "
                     "zavevik llama)")
+    ap.add_argument("--recurrent-compare", action="store_true", help="the same comparison for the family of matrix "
+                    "memories beside a block-local attention: Besulix beside Zavevik (the closest family: a token-by-token "
+                    "recurrence next to attention) and LLaMA")
     ap.add_argument("--hybrid-sizes", nargs="*", default=["2k", "4k"])
     ap.add_argument("--hybrid-families", nargs="*", default=["zavevik", "llama"])
     ap.add_argument("--hybrid-batches", type=int, nargs="*", default=[1, 8])
     args = ap.parse_args()
     if args.latent_compare:
         args.hybrid_families = ["zasevik", "zavevik", "llama"]
+        return _hybrid_compare(args)
+    if args.recurrent_compare:
+        args.hybrid_families = ["besulix", "zavevik", "llama"]
         return _hybrid_compare(args)
     if args.hybrid_compare:
         return _hybrid_compare(args)

@@ -18,28 +18,27 @@
 
 namespace jla {
 
-// grid (M), 256 threads
+// grid (M, ceil(D / 256)), one thread per (token, column): a one-token step is one round trip, not D / 256 of them
 __global__ void __launch_bounds__(256) token_shift_kernel(const float* __restrict__ h, float* prev,
                                                           const float* __restrict__ mu, int n, float* __restrict__ out,
                                                           int S, int D, size_t MD) {
-  const int m = blockIdx.x;
+  const int m = blockIdx.x, d = blockIdx.y * 256 + threadIdx.x;
+  if (d >= D) return;
   const int b = m / S, s = m - b * S;
   const float* cur = h + (size_t)m * D;
   const float* before = s == 0 ? prev + (size_t)b * D : cur - D;
-  const float* last = h + ((size_t)b * S + S - 1) * D;
-  for (int d = threadIdx.x; d < D; d += 256) {
-    const float c = cur[d], diff = before[d] - c;
-    for (int i = 0; i < n; ++i) out[(size_t)i * MD + (size_t)m * D + d] = fmaf(diff, mu[(size_t)i * D + d], c);
-    if (s == 0) prev[(size_t)b * D + d] = last[d];  // (this thread was the only reader of prev[b, d])
-  }
+  const float c = cur[d], diff = before[d] - c;
+  const float last = h[((size_t)b * S + S - 1) * D + d];
+  for (int i = 0; i < n; ++i) out[(size_t)i * MD + (size_t)m * D + d] = fmaf(diff, mu[(size_t)i * D + d], c);
+  if (s == 0) prev[(size_t)b * D + d] = last;  // (this thread was the only reader of prev[b, d])
 }
 
 int hy_token_shift(const float* h, float* prev, const float* mu, int n, float* out, int B, int S, int D, hipStream_t s) {
   if (B < 0 || S < 1 || D < 1 || n < 1) return -1;
   if (B == 0) return 0;
   const long long M = (long long)B * S;
-  if (M > 0x7fffffffLL) return -2;
-  token_shift_kernel<<<(unsigned)M, 256, 0, s>>>(h, prev, mu, n, out, S, D, (size_t)M * D);
+  if (M > 0x7fffffffLL || (D + 255) / 256 > 65535) return -2;
+  token_shift_kernel<<<dim3((unsigned)M, (D + 255) / 256), 256, 0, s>>>(h, prev, mu, n, out, S, D, (size_t)M * D);
   JLA_CHECK_LAUNCH();
   return 0;
 }
@@ -101,29 +100,44 @@ constexpr int LS_PF = LS_STAGE / 256;
 // Staged element i of the chunk starting at token s0. Per token: [k (dimp) | q (dimp) | MODE 1: decay (dimp) |
 // v (cols) | MODE 0: keep, write | pad]; dimp = R slices of LS_PITCH floats (16 values + 4 pad; zeros past dim), cols =
 // the block's state columns [j0, j0 + cols).
+// Staging is split in three so that a thread's 16 loads of a chunk are all in flight together and cost a few
+// instructions each: ls_plan decodes, once per kernel, what the thread's u-th staged element is (its source tensor, its
+// offset inside a token's row, the token within the chunk, what becomes of the loaded number: none of that depends on
+// the chunk); per chunk an address is then one multiply-add on a base chosen by selects (always a readable address, no
+// branch); ls_val turns the loaded number into the staged one when the chunk is written to LDS, a chunk of token
+// steps later.
+enum { LS_ZERO = 0, LS_PLAIN = 1, LS_ONE = 2, LS_DECAY = 3, LS_QUERY = 4 };
+enum { LS_SRC_K = 0, LS_SRC_Q = 1, LS_SRC_D = 2, LS_SRC_V = 3, LS_SRC_KEEP = 4, LS_SRC_WRITE = 5 };
+struct LsPlan {
+  int meta;  // code | source << 3 | token within the chunk << 6
+  int off;   // offset inside the token's row of the source
+};
+
 template <int MODE>
-JLA_DEV float ls_src(const LinScan& p, int b, int h, int s0, int j0, int cols, int dimp, int per, unsigned per_magic,
-                     int i) {
-  const int t = (int)__umulhi((unsigned)i, per_magic), e = i - t * per;  // i / per (exact for i < 2^16)
-  const size_t m = (size_t)b * p.S + s0 + t;
+JLA_DEV LsPlan ls_plan(const LinScan& p, int h, int j0, int cols, int dimp, int per, unsigned per_magic, int i) {
   constexpr int NV = MODE == 1 ? 3 : 2;  // staged vectors over the key rows
-  if (e < NV * dimp) {
-    const int which = e / dimp, ee = e - which * dimp;
-    const int sl = ee / LS_PITCH, w = ee - sl * LS_PITCH, d = sl * LS_SLICE + w;
-    if (w >= LS_SLICE || d >= p.dim) return 0.f;
-    if (which == 0) return p.k[m * p.ldk + (size_t)h * p.dim + d];
-    if (which == 1) return p.q[m * p.ldq + (size_t)h * p.dim + d] * p.q_scale;
-    return expf(-expf(p.decay[m * p.ldd + (size_t)h * p.dim + d] + p.w0[(size_t)h * p.dim + d]));
-  }
-  const int c = e - NV * dimp;
-  if (c < cols) {
-    const int j = j0 + c;
-    if (MODE == 0 && j >= p.vdim) return 1.f;  // the normaliser's column (and surplus columns, never stored)
-    return p.v[m * p.ldv + (size_t)h * p.vdim + min(j, p.vdim - 1)];
-  }
-  if (MODE == 0 && c == cols) return p.decay[m * p.H + h];
-  if (MODE == 0 && c == cols + 1) return p.write[m * p.H + h];
-  return 0.f;
+  const int t = (int)__umulhi((unsigned)i, per_magic), e = i - t * per;  // i / per (exact for i < 2^16)
+  const bool vec = e < NV * dimp;
+  const int which = vec ? e / dimp : 0, ee = vec ? e - which * dimp : 0;
+  const int sl = ee / LS_PITCH, w = ee - sl * LS_PITCH, d = sl * LS_SLICE + w;
+  const bool pad = w >= LS_SLICE || d >= p.dim;
+  const int hd = h * p.dim + (pad ? 0 : d);
+  const int c = e - NV * dimp, j = j0 + c;
+  const bool is_v = !vec && c < cols, is_g = MODE == 0 && !vec && (c == cols || c == cols + 1);
+  const int src = vec ? which : is_v ? LS_SRC_V : is_g ? (c == cols ? LS_SRC_KEEP : LS_SRC_WRITE) : LS_SRC_K;
+  const int code = vec ? (pad ? LS_ZERO : which == 1 ? LS_QUERY : which == 2 ? LS_DECAY : LS_PLAIN)
+                       : is_v ? ((MODE == 0 && j >= p.vdim) ? LS_ONE : LS_PLAIN)  // (the normaliser's column: value 1)
+                              : is_g ? LS_PLAIN : LS_ZERO;
+  LsPlan r;
+  r.meta = code | src << 3 | t << 6;
+  r.off = vec ? hd : is_v ? h * p.vdim + min(max(j, 0), p.vdim - 1) : is_g ? h : h * p.dim;
+  return r;
+}
+
+template <int MODE>
+JLA_DEV float ls_val(int code, float raw, float w0v, float q_scale) {
+  if (MODE == 1 && code == LS_DECAY) return expf(-expf(raw + w0v));
+  return code == LS_ZERO ? 0.f : code == LS_ONE ? 1.f : code == LS_QUERY ? raw * q_scale : raw;
 }
 
 // Sum over the R adjacent lanes that share a column (R a power of two); DPP moves up to 16 lanes.
@@ -160,24 +174,42 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct,
     S[i] = (live && in) ? sp[(size_t)(i0 + i) * ncols] : 0.f;
     uu[i] = (MODE == 1 && in) ? p.u[(size_t)h * p.dim + i0 + i] : 0.f;
   }
-  float pf[LS_PF];
-  {
-    const int n = min(ct, p.S) * per;  // first chunk
+  float pf[LS_PF], pw[LS_PF];
+  LsPlan plan[LS_PF];
+#pragma unroll
+  for (int u = 0; u < LS_PF; ++u) {
+    plan[u] = ls_plan<MODE>(p, h, j0, cols, dimp, per, per_magic, tid + 256 * u);
+    // (the decay's offset does not depend on the token: loaded once)
+    pw[u] = (MODE == 1 && (plan[u].meta & 7) == LS_DECAY) ? p.w0[plan[u].off] : 0.f;
+  }
+  const size_t row0 = (size_t)b * p.S;
+  // loads of the chunk at token sn (n floats of it): every thread issues all of its loads before any is used
+  auto fetch = [&](int sn, int n) {
 #pragma unroll
     for (int u = 0; u < LS_PF; ++u) {
       const int i = tid + 256 * u;
-      if (i < n) stage[i] = ls_src<MODE>(p, b, h, 0, j0, cols, dimp, per, per_magic, i);
+      const int src = (plan[u].meta >> 3) & 7;
+      const size_t m = row0 + sn + (i < n ? plan[u].meta >> 6 : 0);  // (past the chunk: a row of it, never staged)
+      const float* base = src == LS_SRC_K ? p.k : src == LS_SRC_Q ? p.q : src == LS_SRC_V ? p.v
+                          : MODE == 1 ? p.decay : src == LS_SRC_KEEP ? p.decay : p.write;
+      const int ld = src == LS_SRC_K ? p.ldk : src == LS_SRC_Q ? p.ldq : src == LS_SRC_V ? p.ldv : MODE == 1 ? p.ldd : p.H;
+      pf[u] = base[m * ld + plan[u].off];
     }
-  }
+  };
+  auto put = [&](int n) {
+#pragma unroll
+    for (int u = 0; u < LS_PF; ++u) {
+      const int i = tid + 256 * u;
+      if (i < n) stage[i] = ls_val<MODE>(plan[u].meta & 7, pf[u], pw[u], p.q_scale);
+    }
+  };
+  fetch(0, min(ct, p.S) * per);
+  put(min(ct, p.S) * per);
   __syncthreads();
   for (int s0 = 0; s0 < p.S; s0 += ct) {
     const int nt = min(ct, p.S - s0);
     const int nn = min(ct, max(p.S - s0 - ct, 0)) * per;  // next chunk's floats
-#pragma unroll
-    for (int u = 0; u < LS_PF; ++u) {
-      const int i = tid + 256 * u;
-      if (i < nn) pf[u] = ls_src<MODE>(p, b, h, s0 + ct, j0, cols, dimp, per, per_magic, i);
-    }
+    if (nn > 0) fetch(s0 + ct, nn);
     for (int tt = 0; tt < nt; ++tt) {
       const float* row = stage + tt * per;
       const float4* k4 = reinterpret_cast<const float4*>(row + r * LS_PITCH);
@@ -223,11 +255,7 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct,
       if (live && r == 0) p.o[(((size_t)b * p.S + s0 + tt) * p.H + h) * ncols + j] = oq;
     }
     __syncthreads();  // every thread is done reading the chunk
-#pragma unroll
-    for (int u = 0; u < LS_PF; ++u) {
-      const int i = tid + 256 * u;
-      if (i < nn) stage[i] = pf[u];
-    }
+    put(nn);
     __syncthreads();
   }
 #pragma unroll

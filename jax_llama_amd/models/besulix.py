@@ -45,7 +45,7 @@ def cache_specs(config: BesulixConfig) -> list:
     return out
 
 
-def random_state_dict(config: BesulixConfig, seed: int = 0, decay_rank: int = 8) -> Dict[str, torch.Tensor]:
+def random_state_dict(config: BesulixConfig, seed: int = 0, decay_rank: int = 64) -> Dict[str, torch.Tensor]:
     """A random checkpoint of ``config`` with the checkpoint's tensor names (bf16): synthetic benchmarks and tests.
     Scales keep every sublayer's output O(1), the gates away from saturation and the decays spread over (0, 1)."""
     g = torch.Generator().manual_seed(seed)

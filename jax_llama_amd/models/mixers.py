@@ -345,6 +345,7 @@ class TimeMix:
         self.heads, self.dim, self.eps = heads, dim, eps
         self.mu = mu          # fp32 [5, D]: blends of r, k, v, gate, decay
         self.w_rkvg = w_rkvg  # [4, H dim, D]
+        self.w_each = list(w_rkvg.unbind(0))  # (the same four view objects at every call: weight-keyed caches hit)
         self.w_d1, self.w_d2 = w_d1, w_d2  # [rank, D], [H dim, rank]
         self.w0, self.u = w0, u            # fp32 [H, dim]
         self.norm_w = norm_w  # fp32 [H dim]
@@ -358,7 +359,7 @@ class TimeMix:
         if 4 * m <= hy.STACKED_MAX_ROWS:  # a few tokens: the four same-shaped projections as one grouped launch
             r, k, v, g = hy.stacked_linear(mixes[:4], self.w_rkvg).unbind(0)
         else:
-            r, k, v, g = (hy.linear(mixes[j], self.w_rkvg[j]) for j in range(4))
+            r, k, v, g = (hy.linear(mixes[j], self.w_each[j]) for j in range(4))
         wpre = hy.linear(hy.linear(mixes[4], self.w_d1, act=hy.ACT_SOFTCAP, limit=1.0), self.w_d2)
         hd = (nh, dim)
         o = hy.timemix_scan(r.unflatten(1, hd), k.unflatten(1, hd), v.unflatten(1, hd), wpre.unflatten(1, hd), self.w0,

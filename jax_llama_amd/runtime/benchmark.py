@@ -265,9 +265,27 @@ def zasevik_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int,
                                     "embedding": {"scale": width ** 0.5}, "layers": ls})
 
 
+def besulix_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int, layers: int, vocab: int,
+                 chunk: int = 1024, timemix_dim: int = 64):
+    """A Besulix config whose layers have a LLaMA layer's sizes: parallel layers (``heads`` / ``kv_heads`` attention
+    heads of ``head_dim``, half of each q / k head rotated, blocks of ``chunk`` positions, beside ``width /
+    timemix_dim`` time-mix heads of ``timemix_dim``; dense feed-forward of ``ffn``) alternating with matrix-memory
+    layers (``heads`` heads of ``head_dim`` keys and values, no feed-forward)."""
+    from ..config import BesulixConfig
+    left = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5,
+                rot={"base": 1e4, "dims": head_dim // 2}, mask={"size": chunk})
+    par = {"left": left, "right": {"heads": max(1, width // timemix_dim), "dim": timemix_dim}, "left_scale": 0.7,
+           "right_scale": 0.7}
+    mls = dict(heads=heads, dim=head_dim, vdim=head_dim, gate_cap=15.0)
+    ls = [{"type": "mlstm", "mixer": dict(mls), "mlp": None} if i % 2 else
+          {"type": "parallel", "mixer": par, "mlp": {"kind": "dense", "ff": ffn, "limit": 7.0}} for i in range(layers)]
+    return BesulixConfig.from_dict({"architecture": "Besulix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "logit_softcap": 30.0, "layers": ls})
+
+
 def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: int = 64, batches=(1, 8),
                    families=("zavevik", "llama"), progress=lambda m: None) -> Dict[str, object]:
-    """Prefill and decode throughput of the layer-list families (Zavevik, Zasevik) beside LLaMA at equal layer sizes
+    """Prefill and decode throughput of the layer-list families (Zavevik, Zasevik, Besulix) beside LLaMA at equal layer sizes
     (random weights, bf16, synthetic ids), all through the decode engine: ``prefill_tokens_per_sec`` of one warm ``prompt_len``-token prompt per row
     and hipGraph-replayed ``decode_ms_per_token`` over ``gen_len`` steps behind it."""
     from ..config import LLaMAConfig
@@ -284,6 +302,9 @@ def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: 
             elif family == "zasevik":
                 from ..models.zasevik import ZasevikForCausalLM
                 model = ZasevikForCausalLM(zasevik_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
+            elif family == "besulix":
+                from ..models.besulix import BesulixForCausalLM
+                model = BesulixForCausalLM(besulix_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
             else:
                 cfg = LLaMAConfig(vocab_size=sz["vocab"], hidden_size=sz["width"], intermediate_size=sz["ffn"],
                                   num_hidden_layers=sz["layers"], num_attention_heads=sz["heads"],
