@@ -1,7 +1,8 @@
 """jax_llama_amd — an MI355X-native (gfx950 / CDNA4) LLaMA-1/2/3 inference framework with the
 public API of LSaldyt/JAX_llama (reference ``jax_llama/__init__.py:4-10``), plus a model registry with a second
 family (Zavevik: gated delta rule + biased attention + table-routed experts) and a third (Zasevik: latent attention
-with a softmax sink + dense / score-routed feed-forwards) on the same layer-list step function.
+with a softmax sink + dense / score-routed feed-forwards) and a fourth (Besulix: matrix memories + block-local rotary
+attention beside a time-mix recurrence) on the same layer-list step function.
 
 Framework layer: PyTorch-ROCm. Hot path: hand-written HIP kernels (``csrc/kernels``).
 Multi-GPU: one process per GPU, RCCL + a custom xGMI all-reduce. Decode: hipGraph replay.
