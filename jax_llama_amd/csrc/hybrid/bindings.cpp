@@ -193,6 +193,10 @@ void cast_bf16(Tensor x, Tensor y) {
   rc(jla::hy_cast_bf16(f32(x, "x"), reinterpret_cast<jla::bf16_t*>(y.data_ptr()), x.numel(), stream()), "cast_bf16");
 }
 
+void softcap(Tensor x, double cap) {
+  rc(jla::hy_softcap(f32w(x, "x"), x.numel(), (float)cap, stream()), "softcap");
+}
+
 void gelu_gate_rows(Tensor gp, Tensor ids, Tensor table, int64_t col0, Tensor g) {
   const int wb = wtype(table, "table");
   check(gp.dim() == 2 && table.dim() == 2 && g.sizes() == gp.sizes(), "gelu_gate_rows shapes");
@@ -544,6 +548,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("norm_residual", &norm_residual);
   m.def("gelu_gate_rows", &gelu_gate_rows);
   m.def("cast_bf16", &cast_bf16);
+  m.def("softcap", &softcap);
   m.def("attn_prep", &attn_prep);
   m.def("attn_decode_splits", &attn_decode_splits);
   m.def("attn_bias", &attn_bias, py::arg("q"), py::arg("kc"), py::arg("vc"), py::arg("slot"), py::arg("scale"),

@@ -86,6 +86,9 @@ int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_
 typedef uint16_t bf16_t;
 int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s);
 
+// x <- cap * tanh(x / cap) in place (cap = 1: tanh), n elements
+int hy_softcap(float* x, long long n, float cap, hipStream_t s);
+
 // g[m, c] = gelu_tanh(gp[m, c]) * table[ids[m], col0 + c]
 int hy_gelu_gate_rows(const float* gp, const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0,
                       float* g, int M, int D, hipStream_t s);

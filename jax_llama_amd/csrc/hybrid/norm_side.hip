@@ -131,6 +131,21 @@ int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s) {
   return 0;
 }
 
+// x <- cap * tanh(x / cap), one thread per element
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ x, long long n, float cap, float inv_cap) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] * inv_cap);
+}
+
+int hy_softcap(float* x, long long n, float cap, hipStream_t s) {
+  if (n < 0 || !(cap > 0.f)) return -1;
+  if (n == 0) return 0;
+  if ((n + 255) / 256 > 0x7fffffffLL) return -2;
+  softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, n, cap, 1.f / cap);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
 JLA_DEV float ns_gelu_tanh(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }

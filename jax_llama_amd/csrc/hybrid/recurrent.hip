@@ -151,9 +151,17 @@ JLA_DEV float ls_group_sum(float v, int R) {
   return v;
 }
 
-// grid (ceil(ncols * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (power of 2)
-template <int MODE>
-__global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct, int per, unsigned per_magic) {
+// floats of one staged token, tokens per staged chunk
+constexpr int ls_per(int mode, int R) { return ((mode == 1 ? 3 : 2) * R * LS_PITCH + 256 / R + 2 + 3) / 4 * 4; }
+constexpr int ls_ct(int mode, int R) { return LS_STAGE / ls_per(mode, R) < 32 ? LS_STAGE / ls_per(mode, R) : 32; }
+
+// grid (ceil(ncols * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (a power of
+// two, a template parameter: the staged layout, the chunk length and the lane exchange are then compile-time, which took
+// a token step from about 200 instructions to what the state update and the read-out need)
+template <int MODE, int R>
+__global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
+  constexpr int per = ls_per(MODE, R), ct = ls_ct(MODE, R);
+  constexpr unsigned per_magic = (unsigned)((0x100000000ull + per - 1) / per);  // ceil(2^32 / per)
   __shared__ __attribute__((aligned(16))) float stage[LS_STAGE];
   const int ncols = MODE == 0 ? p.vdim + 1 : p.vdim;
   const int tid = threadIdx.x;
@@ -163,8 +171,8 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct,
   const bool live = j < ncols;  // (dead threads still join the lane exchanges)
   const int jc = live ? j : 0;
   const int i0 = r * LS_SLICE;
-  const int j0 = blockIdx.x * (256 / R), cols = 256 / R, jl = j - j0;
-  const int dimp = R * LS_PITCH;
+  constexpr int cols = 256 / R, dimp = R * LS_PITCH;
+  const int j0 = blockIdx.x * cols, jl = j - j0;
   constexpr int NV = MODE == 1 ? 3 : 2;
   float S[LS_SLICE], uu[LS_SLICE];
   float* sp = p.state + (((size_t)b * p.H + h) * p.dim) * ncols + jc;
@@ -206,6 +214,8 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct,
   fetch(0, min(ct, p.S) * per);
   put(min(ct, p.S) * per);
   __syncthreads();
+  float* orow = p.o + (((size_t)b * p.S) * p.H + h) * ncols + jc;  // this column's read-out of the next token
+  const size_t ostride = (size_t)p.H * ncols;
   for (int s0 = 0; s0 < p.S; s0 += ct) {
     const int nt = min(ct, p.S - s0);
     const int nn = min(ct, max(p.S - s0 - ct, 0)) * per;  // next chunk's floats
@@ -252,7 +262,8 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, int R, int ct,
         o0 = fmaf(b0 + b1, v, o0);
       }
       const float oq = ls_group_sum(o0 + o1, R);
-      if (live && r == 0) p.o[(((size_t)b * p.S + s0 + tt) * p.H + h) * ncols + j] = oq;
+      if (live && r == 0) *orow = oq;
+      orow += ostride;
     }
     __syncthreads();  // every thread is done reading the chunk
     put(nn);
@@ -274,15 +285,26 @@ int hy_lin_scan(const LinScan& p, hipStream_t s) {
   if (p.H > 65535 || p.B > 65535) return -3;
   int R = 1;
   while (R * LS_SLICE < p.dim) R <<= 1;
-  const int nv = p.mode == 1 ? 3 : 2;
-  const int per = (nv * R * LS_PITCH + 256 / R + 2 + 3) / 4 * 4;
-  if (per > LS_STAGE) return -4;
-  const int ct = LS_STAGE / per < 32 ? LS_STAGE / per : 32;
   const long long threads = (long long)(p.mode == 0 ? p.vdim + 1 : p.vdim) * R;
-  const unsigned per_magic = (unsigned)((0x100000000ull + per - 1) / per);  // ceil(2^32 / per)
   const dim3 grid((unsigned)((threads + 255) / 256), p.H, p.B);
-  if (p.mode == 0) lin_scan_kernel<0><<<grid, 256, 0, s>>>(p, R, ct, per, per_magic);
-  else lin_scan_kernel<1><<<grid, 256, 0, s>>>(p, R, ct, per, per_magic);
+#define LS_LAUNCH(RR)                                                   \
+  case RR:                                                              \
+    static_assert(ls_per(1, RR) <= LS_STAGE, "a staged token fits");    \
+    if (p.mode == 0) lin_scan_kernel<0, RR><<<grid, 256, 0, s>>>(p);    \
+    else lin_scan_kernel<1, RR><<<grid, 256, 0, s>>>(p);                \
+    break
+  switch (R) {
+    LS_LAUNCH(1);
+    LS_LAUNCH(2);
+    LS_LAUNCH(4);
+    LS_LAUNCH(8);
+    LS_LAUNCH(16);
+    LS_LAUNCH(32);
+    LS_LAUNCH(64);
+    default:
+      return -4;
+  }
+#undef LS_LAUNCH
   JLA_CHECK_LAUNCH();
   return 0;
 }

@@ -360,7 +360,7 @@ class TimeMix:
             r, k, v, g = hy.stacked_linear(mixes[:4], self.w_rkvg).unbind(0)
         else:
             r, k, v, g = (hy.linear(mixes[j], self.w_each[j]) for j in range(4))
-        wpre = hy.linear(hy.linear(mixes[4], self.w_d1, act=hy.ACT_SOFTCAP, limit=1.0), self.w_d2)
+        wpre = hy.linear(hy.linear_softcap(mixes[4], self.w_d1, 1.0), self.w_d2)
         hd = (nh, dim)
         o = hy.timemix_scan(r.unflatten(1, hd), k.unflatten(1, hd), v.unflatten(1, hd), wpre.unflatten(1, hd), self.w0,
                             self.u, state, ctx.b, ctx.s)

@@ -424,6 +424,23 @@ def rms_rows(y: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (fp32, contiguous; ``cap = 1``: a tanh)."""
+    if not _gpu(x):
+        return x.copy_(cap * torch.tanh(x.float() / cap))
+    ext().softcap(x, float(cap))
+    return x
+
+
+def linear_softcap(x, w: torch.Tensor, cap: float) -> torch.Tensor:
+    """``cap * tanh((x @ w^T) / cap)``: in the linear's epilogue, or, where a prompt-sized product runs on the packed MFMA
+    GEMM (which has no such epilogue), as one elementwise pass behind it: a product with a few dozen output columns is
+    a handful of tiles for the row-major kernel and a split-K plan for the packed one."""
+    if _gpu(w) and not isinstance(x, RmsInput) and _use_packed_gemm(x, w):
+        return softcap_(linear(x, w), cap)
+    return linear(x, w, act=ACT_SOFTCAP, limit=cap)
+
+
 def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z * z * z)))
 

@@ -71,9 +71,9 @@ def cfg_odd():
             ]}
 
 
-def build(cfg, device, dtype=F32, seed=0, edit=None):
+def build(cfg, device, dtype=F32, seed=0, edit=None, decay_rank=5):
     config = BesulixConfig.from_dict(cfg)
-    sd = random_state_dict(config, seed=seed, decay_rank=5)
+    sd = random_state_dict(config, seed=seed, decay_rank=decay_rank)
     for k in list(sd):
         if k.endswith("mlp.gate") or k.endswith("mlp.up"):  # pre-activations on both sides of the clamps
             sd[k] = (sd[k].float() * 2.0).to(BF16)
@@ -355,6 +355,9 @@ def test_soft_capped_linear(device):
     x, w = torch.randn(9, 40, generator=g) * 3.0, torch.randn(24, 40, generator=g)
     ref = 2.5 * np.tanh(x.double().numpy() @ w.double().numpy().T / 2.5)
     assert err(hy.linear(x.to(device), w.to(device), act=hy.ACT_SOFTCAP, limit=2.5).cpu().numpy(), ref) < 2e-5
+    assert err(hy.linear_softcap(x.to(device), w.to(device), 2.5).cpu().numpy(), ref) < 2e-5
+    y = (x @ w.t()).to(device).contiguous()
+    assert err(hy.softcap_(y, 2.5).cpu().numpy(), ref) < 2e-5
 
 
 # ---------------------------------------------------------------------------------------------- whole model
@@ -563,7 +566,7 @@ def test_longer_prompts_at_the_kernel_shapes(dtype):
     block edges inside a wave's queries, decode over several key runs) on the GPU against the framework's fp32 CPU path,
     which the tests above tie to the oracle."""
     cfg = cfg_kernel_shapes()
-    ref_model, sd = build(cfg, "cpu", F32)
+    ref_model, sd = build(cfg, "cpu", F32, decay_rank=32)  # (a rank the packed GEMM takes: its soft cap is a pass of its own)
     t = toks(600, 300, seed=21)
     with torch.no_grad():
         ref = ref_model(torch.tensor([t], dtype=torch.int32)).logits[0].numpy()
