@@ -500,7 +500,7 @@ void mlstm_prep(Tensor proj, int64_t col_i, int64_t col_f, Tensor gate_bias, dou
 }
 
 void lin_scan(int64_t mode, Tensor q, Tensor k, Tensor v, Tensor decay, OptT write, OptT w0, OptT u, Tensor state,
-              Tensor o, int64_t B, int64_t S, double q_scale) {
+              Tensor o, int64_t B, int64_t S, double q_scale, int64_t nseg, int64_t seg_len, OptT seg_ws) {
   jla::LinScan p{};
   check(mode == 0 || mode == 1, "lin_scan: mode");
   check(q.dim() == 3 && v.dim() == 3, "lin_scan: q, k are [M, H, dim], v is [M, H, vdim]");
@@ -525,6 +525,15 @@ void lin_scan(int64_t mode, Tensor q, Tensor k, Tensor v, Tensor decay, OptT wri
   p.o = f32w(o, "o");
   p.B = B; p.S = S; p.H = H; p.dim = dim; p.vdim = vdim;
   p.q_scale = q_scale;
+  check(nseg >= 1 && seg_len >= 1 && nseg * seg_len >= S && (nseg - 1) * seg_len < S, "lin_scan: segments cover the tokens");
+  p.nseg = nseg;
+  p.seg_len = seg_len;
+  if (nseg > 1) {
+    const int64_t ns = B * nseg * H * dim * cols, nd = B * nseg * H * (mode == 1 ? dim : 1);
+    check(seg_ws.has_value() && seg_ws->numel() >= ns + nd, "lin_scan: segment workspace");
+    p.seg_state = f32w(*seg_ws, "seg_ws");
+    p.seg_decay = p.seg_state + ns;
+  }
   rc(jla::hy_lin_scan(p, stream()), "lin_scan");
 }
 
@@ -566,5 +575,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rotate_heads", &rotate_heads);
   m.def("token_shift", &token_shift);
   m.def("mlstm_prep", &mlstm_prep);
-  m.def("lin_scan", &lin_scan);
+  m.def("lin_scan", &lin_scan, py::arg("mode"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("decay"),
+        py::arg("write"), py::arg("w0"), py::arg("u"), py::arg("state"), py::arg("o"), py::arg("B"), py::arg("S"),
+        py::arg("q_scale"), py::arg("nseg") = 1, py::arg("seg_len") = (int64_t)1 << 40, py::arg("seg_ws") = py::none());
 }

@@ -264,6 +264,13 @@ struct LinScan {
   float* o;  // [M, H, cols]
   int B, S, H, dim, vdim;
   float q_scale;
+  // nseg > 1: the sequence runs as nseg segments of seg_len tokens side by side (every segment non-empty), in three
+  // launches (each segment's own final state and decay product, their combination, the scan proper from each segment's
+  // incoming state); seg_state holds B * nseg * H * dim * cols floats, seg_decay B * nseg * H (* dim in mode 1).
+  // nseg == 1 (seg_len >= S): one launch.
+  int nseg, seg_len;
+  float* seg_state;
+  float* seg_decay;
 };
 int hy_lin_scan(const LinScan& p, hipStream_t s);
 

@@ -158,15 +158,22 @@ constexpr int ls_ct(int mode, int R) { return LS_STAGE / ls_per(mode, R) < 32 ? 
 // grid (ceil(ncols * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (a power of
 // two, a template parameter: the staged layout, the chunk length and the lane exchange are then compile-time, which took
 // a token step from about 200 instructions to what the state update and the read-out need)
-template <int MODE, int R>
-__global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
+//
+// A long sequence is cut into nseg segments that run side by side (grid.z = B * nseg), in three launches: (1) STATE_ONLY:
+// every segment from a zero state, no read-out, leaving its final state T and the product D of its decays; (2)
+// lin_combine_kernel walks the segments once, S_in(p + 1) = D_p S_in(p) + T_p from the carried state, and stores the
+// sequence's final state; (3) the full scan of every segment from its S_in. A token's arithmetic inside a segment is that
+// of the one-launch form; the incoming state is a two-term sum instead of a running one.
+template <int MODE, int R, int STATE_ONLY>
+__global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p, const float* s_init, float* s_final, float* seg_decay) {
   constexpr int per = ls_per(MODE, R), ct = ls_ct(MODE, R);
   constexpr unsigned per_magic = (unsigned)((0x100000000ull + per - 1) / per);  // ceil(2^32 / per)
   __shared__ __attribute__((aligned(16))) float stage[LS_STAGE];
   const int ncols = MODE == 0 ? p.vdim + 1 : p.vdim;
   const int tid = threadIdx.x;
   const int t = blockIdx.x * 256 + tid;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.y, b = blockIdx.z / p.nseg, seg = blockIdx.z - b * p.nseg;
+  const int t_lo = seg * p.seg_len, t_hi = min(p.S, t_lo + p.seg_len);  // this block's tokens
   const int j = t / R, r = t - j * R;
   const bool live = j < ncols;  // (dead threads still join the lane exchanges)
   const int jc = live ? j : 0;
@@ -174,14 +181,16 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
   constexpr int cols = 256 / R, dimp = R * LS_PITCH;
   const int j0 = blockIdx.x * cols, jl = j - j0;
   constexpr int NV = MODE == 1 ? 3 : 2;
-  float S[LS_SLICE], uu[LS_SLICE];
-  float* sp = p.state + (((size_t)b * p.H + h) * p.dim) * ncols + jc;
+  float S[LS_SLICE], uu[LS_SLICE], dprod[MODE == 1 ? LS_SLICE : 1];
+  const size_t sidx = ((((size_t)b * p.nseg + seg) * p.H + h) * p.dim) * ncols + jc;  // (b, segment, head) of a state array
 #pragma unroll
   for (int i = 0; i < LS_SLICE; ++i) {
     const bool in = i0 + i < p.dim;
-    S[i] = (live && in) ? sp[(size_t)(i0 + i) * ncols] : 0.f;
+    S[i] = (s_init && live && in) ? s_init[sidx + (size_t)(i0 + i) * ncols] : 0.f;
     uu[i] = (MODE == 1 && in) ? p.u[(size_t)h * p.dim + i0 + i] : 0.f;
+    if (MODE == 1) dprod[i] = 1.f;
   }
+  if (MODE == 0) dprod[0] = 1.f;
   float pf[LS_PF], pw[LS_PF];
   LsPlan plan[LS_PF];
 #pragma unroll
@@ -211,14 +220,14 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
       if (i < n) stage[i] = ls_val<MODE>(plan[u].meta & 7, pf[u], pw[u], p.q_scale);
     }
   };
-  fetch(0, min(ct, p.S) * per);
-  put(min(ct, p.S) * per);
+  fetch(t_lo, min(ct, t_hi - t_lo) * per);
+  put(min(ct, t_hi - t_lo) * per);
   __syncthreads();
-  float* orow = p.o + (((size_t)b * p.S) * p.H + h) * ncols + jc;  // this column's read-out of the next token
+  float* orow = p.o + (((size_t)b * p.S + t_lo) * p.H + h) * ncols + jc;  // this column's read-out of the next token
   const size_t ostride = (size_t)p.H * ncols;
-  for (int s0 = 0; s0 < p.S; s0 += ct) {
-    const int nt = min(ct, p.S - s0);
-    const int nn = min(ct, max(p.S - s0 - ct, 0)) * per;  // next chunk's floats
+  for (int s0 = t_lo; s0 < t_hi; s0 += ct) {
+    const int nt = min(ct, t_hi - s0);
+    const int nn = min(ct, max(t_hi - s0 - ct, 0)) * per;  // next chunk's floats
     if (nn > 0) fetch(s0 + ct, nn);
     for (int tt = 0; tt < nt; ++tt) {
       const float* row = stage + tt * per;
@@ -235,12 +244,15 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
       float o0 = 0.f, o1 = 0.f;
       if (MODE == 0) {
         const float keep = row[NV * dimp + cols], wv = row[NV * dimp + cols + 1] * v;
+        if (STATE_ONLY) dprod[0] *= keep;
 #pragma unroll
         for (int i = 0; i < LS_SLICE; i += 2) {
           S[i] = fmaf(keep, S[i], kv[i] * wv);
           S[i + 1] = fmaf(keep, S[i + 1], kv[i + 1] * wv);
-          o0 = fmaf(S[i], qv[i], o0);
-          o1 = fmaf(S[i + 1], qv[i + 1], o1);
+          if (!STATE_ONLY) {
+            o0 = fmaf(S[i], qv[i], o0);
+            o1 = fmaf(S[i + 1], qv[i + 1], o1);
+          }
         }
       } else {
         const float4* d4 = reinterpret_cast<const float4*>(row + 2 * dimp + r * LS_PITCH);
@@ -252,26 +264,65 @@ __global__ void __launch_bounds__(256) lin_scan_kernel(LinScan p) {
         }
 #pragma unroll
         for (int i = 0; i < LS_SLICE; i += 2) {
-          o0 = fmaf(S[i], qv[i], o0);
-          o1 = fmaf(S[i + 1], qv[i + 1], o1);
-          b0 = fmaf(uu[i] * kv[i], qv[i], b0);
-          b1 = fmaf(uu[i + 1] * kv[i + 1], qv[i + 1], b1);
+          if (!STATE_ONLY) {
+            o0 = fmaf(S[i], qv[i], o0);
+            o1 = fmaf(S[i + 1], qv[i + 1], o1);
+            b0 = fmaf(uu[i] * kv[i], qv[i], b0);
+            b1 = fmaf(uu[i + 1] * kv[i + 1], qv[i + 1], b1);
+          } else {
+            dprod[i] *= dv[i];
+            dprod[i + 1] *= dv[i + 1];
+          }
           S[i] = fmaf(dv[i], S[i], kv[i] * v);
           S[i + 1] = fmaf(dv[i + 1], S[i + 1], kv[i + 1] * v);
         }
         o0 = fmaf(b0 + b1, v, o0);
       }
-      const float oq = ls_group_sum(o0 + o1, R);
-      if (live && r == 0) *orow = oq;
-      orow += ostride;
+      if (!STATE_ONLY) {
+        const float oq = ls_group_sum(o0 + o1, R);
+        if (live && r == 0) *orow = oq;
+        orow += ostride;
+      }
     }
     __syncthreads();  // every thread is done reading the chunk
     put(nn);
     __syncthreads();
   }
+  if (s_final) {
 #pragma unroll
-  for (int i = 0; i < LS_SLICE; ++i)
-    if (live && i0 + i < p.dim) sp[(size_t)(i0 + i) * ncols] = S[i];
+    for (int i = 0; i < LS_SLICE; ++i)
+      if (live && i0 + i < p.dim) s_final[sidx + (size_t)(i0 + i) * ncols] = S[i];
+  }
+  if (STATE_ONLY && seg_decay && j == 0) {  // the segment's decay: one number per head, or one per key row
+    const size_t d0 = ((size_t)b * p.nseg + seg) * p.H + h;
+    if (MODE == 0) {
+      if (r == 0) seg_decay[d0] = dprod[0];
+    } else {
+#pragma unroll
+      for (int i = 0; i < LS_SLICE; ++i)
+        if (i0 + i < p.dim) seg_decay[d0 * p.dim + i0 + i] = dprod[MODE == 1 ? i : 0];
+    }
+  }
+}
+
+// one thread per state element of a (row, head): on entry seg[b][s] holds segment s's own final state, on exit the
+// state segment s starts from; state (the carried one) is advanced past the whole sequence
+__global__ void __launch_bounds__(256) lin_combine_kernel(float* state, float* seg, const float* seg_decay, int nseg,
+                                                          int H, int dim, int ncols, int per_row_decay, long long n) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;  // element of [B, H, dim, ncols]
+  if (e >= n) return;
+  const long long hsz = (long long)dim * ncols, bh = e / hsz, in = e - bh * hsz;
+  const long long b = bh / H, h = bh - b * H;
+  const int row = (int)(in / ncols);
+  float S = state[e];
+  for (int s = 0; s < nseg; ++s) {
+    const long long at = ((b * nseg + s) * H + h) * hsz + in;
+    const long long dh = (b * nseg + s) * H + h;
+    const float d = seg_decay[per_row_decay ? dh * dim + row : dh], own = seg[at];
+    seg[at] = S;
+    S = fmaf(d, S, own);
+  }
+  state[e] = S;
 }
 
 int hy_lin_scan(const LinScan& p, hipStream_t s) {
@@ -286,23 +337,47 @@ int hy_lin_scan(const LinScan& p, hipStream_t s) {
   int R = 1;
   while (R * LS_SLICE < p.dim) R <<= 1;
   const long long threads = (long long)(p.mode == 0 ? p.vdim + 1 : p.vdim) * R;
-  const dim3 grid((unsigned)((threads + 255) / 256), p.H, p.B);
-#define LS_LAUNCH(RR)                                                   \
-  case RR:                                                              \
-    static_assert(ls_per(1, RR) <= LS_STAGE, "a staged token fits");    \
-    if (p.mode == 0) lin_scan_kernel<0, RR><<<grid, 256, 0, s>>>(p);    \
-    else lin_scan_kernel<1, RR><<<grid, 256, 0, s>>>(p);                \
+  const int ncols = p.mode == 0 ? p.vdim + 1 : p.vdim;
+  const bool cut = p.nseg > 1;
+  if (cut && (!p.seg_state || !p.seg_decay || p.seg_len < 1 || (long long)p.nseg * p.seg_len < p.S ||
+              (long long)(p.nseg - 1) * p.seg_len >= p.S))
+    return -7;
+  if (!cut && (p.nseg != 1 || p.seg_len < p.S)) return -7;
+  if ((long long)p.B * p.nseg > 65535) return -3;
+  const dim3 grid((unsigned)((threads + 255) / 256), p.H, p.B * p.nseg);
+#define LS_LAUNCH(RR)                                                                                            \
+  case RR:                                                                                                       \
+    static_assert(ls_per(1, RR) <= LS_STAGE, "a staged token fits");                                             \
+    if (!cut) {                                                                                                  \
+      if (p.mode == 0) lin_scan_kernel<0, RR, 0><<<grid, 256, 0, s>>>(p, p.state, p.state, nullptr);             \
+      else lin_scan_kernel<1, RR, 0><<<grid, 256, 0, s>>>(p, p.state, p.state, nullptr);                         \
+    } else if (pass == 0) {                                                                                      \
+      if (p.mode == 0) lin_scan_kernel<0, RR, 1><<<grid, 256, 0, s>>>(p, nullptr, p.seg_state, p.seg_decay);     \
+      else lin_scan_kernel<1, RR, 1><<<grid, 256, 0, s>>>(p, nullptr, p.seg_state, p.seg_decay);                 \
+    } else {                                                                                                     \
+      if (p.mode == 0) lin_scan_kernel<0, RR, 0><<<grid, 256, 0, s>>>(p, p.seg_state, nullptr, nullptr);         \
+      else lin_scan_kernel<1, RR, 0><<<grid, 256, 0, s>>>(p, p.seg_state, nullptr, nullptr);                     \
+    }                                                                                                            \
     break
-  switch (R) {
-    LS_LAUNCH(1);
-    LS_LAUNCH(2);
-    LS_LAUNCH(4);
-    LS_LAUNCH(8);
-    LS_LAUNCH(16);
-    LS_LAUNCH(32);
-    LS_LAUNCH(64);
-    default:
-      return -4;
+  for (int pass = 0; pass < (cut ? 2 : 1); ++pass) {
+    switch (R) {
+      LS_LAUNCH(1);
+      LS_LAUNCH(2);
+      LS_LAUNCH(4);
+      LS_LAUNCH(8);
+      LS_LAUNCH(16);
+      LS_LAUNCH(32);
+      LS_LAUNCH(64);
+      default:
+        return -4;
+    }
+    JLA_CHECK_LAUNCH();
+    if (cut && pass == 0) {
+      const long long n = (long long)p.B * p.H * p.dim * ncols;
+      lin_combine_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p.state, p.seg_state, p.seg_decay, p.nseg, p.H, p.dim,
+                                                                    ncols, p.mode == 1, n);
+      JLA_CHECK_LAUNCH();
+    }
   }
 #undef LS_LAUNCH
   JLA_CHECK_LAUNCH();

@@ -826,6 +826,28 @@ def mlstm_prep(proj: torch.Tensor, col_i: int, col_f: int, gate_bias: torch.Tens
     return out[0], out[1], out[2]
 
 
+# A prompt's recurrence runs as several segments side by side when one pass would leave most of the chip idle: segments
+# of at least SCAN_SEG_MIN tokens, as many as bring the launch to about SCAN_TARGET_BLOCKS workgroups.
+SCAN_SEG_MIN = 64
+SCAN_TARGET_BLOCKS = int(os.environ.get("JLA_HY_SCAN_BLOCKS", "1024"))
+
+
+def _scan_segments(b: int, s: int, heads: int, dim: int, cols: int, device):
+    """``(nseg, seg_len, workspace)`` of a scan over ``s`` tokens of ``b`` rows (csrc/hybrid/recurrent.hip: a thread
+    holds 16 key rows of a state column, 256 threads a workgroup)."""
+    lanes = 1
+    while lanes * 16 < dim:
+        lanes *= 2
+    blocks = b * heads * ((cols * lanes + 255) // 256)
+    nseg = min(s // SCAN_SEG_MIN, SCAN_TARGET_BLOCKS // max(1, blocks))
+    if nseg < 2:
+        return 1, max(s, 1), None
+    seg_len = (s + nseg - 1) // nseg
+    nseg = (s + seg_len - 1) // seg_len
+    ws = torch.empty(b * nseg * heads * dim * (cols + 1), dtype=F32, device=device)
+    return nseg, seg_len, ws
+
+
 def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, keep: torch.Tensor, write: torch.Tensor,
                state: torch.Tensor, b: int, s: int, q_scale: float = 1.0) -> torch.Tensor:
     """Matrix memory with scalar gates per head, read after the write. ``q, k [M, H, dim]``, ``v [M, H, vdim]`` (column
@@ -846,7 +868,8 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, keep: torch.Te
             o[:, t] = torch.einsum("bhdv,bhd->bhv", state, qq[:, t])
         return o.reshape(m, h, vdim + 1)
     o = torch.empty(m, h, vdim + 1, dtype=F32, device=q.device)
-    ext().lin_scan(0, q, k, v, keep, write, None, None, state, o, b, s, float(q_scale))
+    nseg, seg_len, ws = _scan_segments(b, s, h, dim, vdim + 1, q.device)
+    ext().lin_scan(0, q, k, v, keep, write, None, None, state, o, b, s, float(q_scale), nseg, seg_len, ws)
     return o
 
 
@@ -871,5 +894,6 @@ def timemix_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wpre: torch.
             state.add_(kv)
         return o.reshape(m, h, vdim)
     o = torch.empty(m, h, vdim, dtype=F32, device=r.device)
-    ext().lin_scan(1, r, k, v, wpre, None, w0.reshape(h, dim), u.reshape(h, dim), state, o, b, s, 1.0)
+    nseg, seg_len, ws = _scan_segments(b, s, h, dim, vdim, r.device)
+    ext().lin_scan(1, r, k, v, wpre, None, w0.reshape(h, dim), u.reshape(h, dim), state, o, b, s, 1.0, nseg, seg_len, ws)
     return o

@@ -312,6 +312,35 @@ def test_time_mix_mechanism(device, heads, dim, rank):
         assert err(run_mixer(mixer, cache, h, portions, device), ref) < 2e-5, portions
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seg_min", [4, 8, 16])
+def test_scans_cut_into_segments(seg_min, monkeypatch):
+    """Both recurrences with a prompt's tokens dealt to segments that run side by side (each segment's own final state
+    and decay product, their combination from the carried state, then the scan proper): many short segments, an uneven
+    last one, a second portion that starts from a carried state, against the oracle."""
+    monkeypatch.setattr(hy, "SCAN_SEG_MIN", seg_min)
+    t, d, eps, device = 75, 48, 1e-6, "cuda"
+    g = torch.Generator().manual_seed(11)
+    h = torch.randn(t, d, generator=g)
+    for heads, dim, vdim, cap in [(3, 8, 12, 4.0), (2, 40, 33, 9.0), (1, 130, 4, 2.0)]:
+        w = _mlstm_weights(g, heads, dim, vdim, d, 1.0)
+        ref = ob.mlstm(w, "m.", _mls(heads, dim, vdim, cap), h.double().numpy(), eps)
+        for portions in ([75], [40, 35], [9, 66]):
+            assert hy._scan_segments(1, portions[-1], heads, dim, vdim + 1, device)[0] > 1
+            cache = HybridCache([("mlstm", heads, dim, vdim)], 1, t, device, F32)
+            mixer = MatrixLSTM(0, heads, dim, vdim, cap, eps,
+                               torch.cat([w["m." + n] for n in ("q", "k", "v", "g", "i", "f")]).to(device),
+                               torch.cat([w["m.i.b"], w["m.f.b"]]).to(device), w["m.norm"].to(device), w["m.o"].to(device))
+            assert err(run_mixer(mixer, cache, h, portions, device), ref) < 2e-5, (heads, dim, portions)
+    for heads, dim, rank in [(3, 8, 5), (2, 40, 7), (1, 136, 4)]:
+        w = _timemix_weights(g, heads, dim, d, rank)
+        ref = ob.time_mix(w, "m.", {"heads": heads, "dim": dim}, h.double().numpy(), eps)
+        for portions in ([75], [40, 35], [9, 66]):
+            cache = HybridCache([("timemix", heads, dim, dim, d)], 1, t, device, F32)
+            assert err(run_mixer(_timemix_mixer(w, heads, dim, d, eps, device), cache, h, portions, device), ref) < 2e-5, \
+                (heads, dim, portions)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_side_by_side_mixers_share_one_projection(device):
     """Attention and time mix on one input, summed with unequal weights through one output projection."""
