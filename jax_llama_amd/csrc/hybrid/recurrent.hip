@@ -54,11 +54,20 @@ __global__ void __launch_bounds__(64) mlstm_prep_kernel(MlstmPrep p) {
   const float bi = p.gate_bias[h], bf = p.gate_bias[p.H + h];
   const float inv_cap = 1.f / p.cap;
   float m = p.mstate[(size_t)b * p.H + h];
+  // this lane's gate pre-activations of the chunk at t0 (a lane past the end re-reads the last token)
+  auto gates = [&](int t0, float& xi, float& xf) {
+    const size_t row = (size_t)b * p.S + min(t0 + lane, p.S - 1);
+    xi = p.proj[row * p.ld + p.col_i + h];
+    xf = p.proj[row * p.ld + p.col_f + h];
+  };
+  float xi_next, xf_next;
+  gates(0, xi_next, xf_next);
   for (int t0 = 0; t0 < p.S; t0 += 64) {
     const int t = t0 + lane;
     const bool on = t < p.S;
     const size_t row = (size_t)b * p.S + (on ? t : p.S - 1);
-    const float xi = p.proj[row * p.ld + p.col_i + h], xf = p.proj[row * p.ld + p.col_f + h];
+    const float xi = xi_next, xf = xf_next;
+    if (t0 + 64 < p.S) gates(t0 + 64, xi_next, xf_next);  // (in flight behind this chunk's chain)
     // (a token past the end keeps m: f = 0, a = -inf)
     const float a = on ? p.cap * tanhf((xi + bi) * inv_cap) : -INFINITY;
     const float f = on ? rc_logsigmoid(p.cap * tanhf((xf + bf) * inv_cap)) : 0.f;
