@@ -1,6 +1,7 @@
 // Host launchers of the hybrid-sequence-mixer kernels (module jax_llama_amd._C_hybrid): row-gathered / expert-grouped
-// linears on row-major weights of any shape, attention with a distance-bias table and a score soft cap, the gated
-// delta rule with its short convolutions, and the output-side norms. Pure HIP translation units (no torch headers).
+// linears on row-major weights of any shape, attention with a distance-bias table and a score soft cap (and block-local
+// masks, sinks, per-head factors), rotary positions, the gated delta rule with its short convolutions, two matrix-memory
+// recurrences with their gates, and the output-side norms. Pure HIP translation units (no torch headers).
 // Every launcher returns 0 on success, <0 on a shape/argument error, >0 for a hipError_t.
 //
 // Activations between kernels are fp32 in both number formats. "wbf16" selects the weight / cache element type: bf16

@@ -12,7 +12,9 @@
 //                    current token (per-channel D from a double exponential: the time-mix memory). Thread layout of the
 //                    delta-rule scan: a thread owns 16 key rows of one state column in registers, the lanes of a column
 //                    combine their partial read-outs by lane exchange, tokens are staged through LDS a chunk at a time
-//                    with the next chunk's loads in flight.
+//                    with the next chunk's loads in flight. A long sequence is cut into segments that run side by side
+//                    (both recurrences are linear in the state): segment states and decay products, one combining
+//                    walk, then the scan proper from every segment's incoming state.
 #include "hy_util.h"
 #include "hybrid.h"
 
