@@ -7,7 +7,7 @@ attention beside a time-mix recurrence) on the same layer-list step function.
 Framework layer: PyTorch-ROCm. Hot path: hand-written HIP kernels (``csrc/kernels``).
 Multi-GPU: one process per GPU, RCCL + a custom xGMI all-reduce. Decode: hipGraph replay.
 """
-from .config import BesulixConfig, LLaMAConfig, ModelArgs, ZasevikConfig, ZavevikConfig, config_from_params, get_preset, swiglu_hidden_size
+from .config import BesulixConfig, LLaMAConfig, ModelArgs, ZasevikConfig, ZavevikConfig, ZifisunConfig, config_from_params, get_preset, swiglu_hidden_size
 from .generation import LLaMA
 from .models import (CausalLMOutput, FlaxLLaMAForCausalLM, FlaxLLaMAModel, KVCache, LLaMAForCausalLM,
                      LLaMAModel)
@@ -16,6 +16,7 @@ from .parallel.partition import (Mesh, P, PartitionSpec, get_llama_param_partiti
 from .models.registry import load_model
 from .models.zasevik import ZasevikForCausalLM
 from .models.besulix import BesulixForCausalLM
+from .models.zifisun import ZifisunForCausalLM
 from .models.zavevik import ZavevikForCausalLM
 from .runtime.engine import GenerationConfig
 from .runtime.stepper import SequenceStepper
@@ -30,5 +31,5 @@ __all__ = [
     "CausalLMOutput", "KVCache", "GenerationConfig",
     "Mesh", "P", "PartitionSpec", "get_llama_param_partition_spec", "with_named_sharding_constraint",
     "with_sharding_constraint", "LLaMA2Tokenizer", "LLaMA3Tokenizer", "ChatFormat", "convert_llama_weights",
-    "ZavevikConfig", "ZavevikForCausalLM", "ZasevikConfig", "ZasevikForCausalLM", "BesulixConfig", "BesulixForCausalLM", "SequenceStepper", "load_model",
+    "ZavevikConfig", "ZavevikForCausalLM", "ZasevikConfig", "ZasevikForCausalLM", "BesulixConfig", "BesulixForCausalLM", "ZifisunConfig", "ZifisunForCausalLM", "SequenceStepper", "load_model",
 ]

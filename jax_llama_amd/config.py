@@ -663,3 +663,221 @@ class BesulixConfig:
 
     def __repr__(self) -> str:
         return f"BesulixConfig {json.dumps(self.to_dict(), sort_keys=True)}"
+
+
+# -------------------------------------------------------------------------------------
+# Zifisun: windowed latent / normed attention, grouped routing with identity experts, several residual streams
+# -------------------------------------------------------------------------------------
+def _mask_from(d: Optional[Dict[str, Any]]):
+    """``(window, keep_first)`` of a mixer's ``mask`` entry (absent: plain causal attention)."""
+    d = d or {}
+    window, keep = int(d.get("size") or 0), int(d.get("keep_first") or 0)
+    if window < 0 or keep < 0:
+        raise ValueError("mask.size and mask.keep_first must not be negative")
+    return window, keep
+
+
+def _mask_to(window: int, keep_first: int) -> Optional[Dict[str, Any]]:
+    if not window:
+        return None
+    return {"size": window, "keep_first": keep_first} if keep_first else {"size": window}
+
+
+@dataclass
+class RotaryLatentSpec:
+    """Latent attention with a query latent and one rotated key part: ``heads`` heads of ``dim`` plain and ``rot_dim``
+    rotated query / key numbers and ``vdim`` value numbers; keys and values come from ``kv_rank`` cached numbers per
+    token, queries from ``q_rank``; rotary base ``rot_base`` over ``rot_dims`` of the rotated part; a query sees the last
+    ``window`` positions (0: all) and the first ``keep_first`` of the sequence."""
+
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot_base: float
+    rot_dims: int
+    window: int = 0
+    keep_first: int = 0
+    type = "latent_attention"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "RotaryLatentSpec":
+        dim, rot_dim = int(d["dim"]), int(d.get("rot_dim", 0) or 0)
+        rot = d.get("rot") or {}
+        window, keep = _mask_from(d.get("mask"))
+        out = cls(heads=int(d["heads"]), dim=dim, rot_dim=rot_dim, vdim=int(d.get("vdim", dim)), kv_rank=int(d["kv_rank"]),
+                  q_rank=int(d["q_rank"]), scale=float(d["scale"]), rot_base=float(rot.get("base", 10000.0)),
+                  rot_dims=int(rot.get("dims", rot_dim)), window=window, keep_first=keep)
+        if out.rot_dims % 2 or out.rot_dims > out.rot_dim:
+            raise ValueError("rot.dims must be even and at most rot_dim")
+        if min(out.heads, out.dim, out.vdim, out.kv_rank, out.q_rank) < 1:
+            raise ValueError("latent_attention: sizes must be positive")
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = dict(heads=self.heads, dim=self.dim, rot_dim=self.rot_dim, vdim=self.vdim,
+                                   kv_rank=self.kv_rank, q_rank=self.q_rank, scale=self.scale,
+                                   rot={"base": self.rot_base, "dims": self.rot_dims})
+        mask = _mask_to(self.window, self.keep_first)
+        if mask:
+            out["mask"] = mask
+        return out
+
+
+@dataclass
+class NormedAttentionSpec:
+    """Softmax attention without positions: ``heads`` query heads over ``kv_heads`` key / value heads, q and k RMS-normed
+    per head with a weight, an output gate per head, a sliding window that may keep the sequence's first keys."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    keep_first: int = 0
+    type = "attention"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "NormedAttentionSpec":
+        heads, dim = int(d["heads"]), int(d["dim"])
+        window, keep = _mask_from(d.get("mask"))
+        out = cls(heads=heads, kv_heads=int(d.get("kv_heads", heads)), dim=dim, vdim=int(d.get("vdim", dim)),
+                  scale=float(d["scale"]), window=window, keep_first=keep)
+        if out.heads % out.kv_heads:
+            raise ValueError("heads must be divisible by kv_heads")
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = dict(heads=self.heads, kv_heads=self.kv_heads, dim=self.dim, vdim=self.vdim, scale=self.scale)
+        mask = _mask_to(self.window, self.keep_first)
+        if mask:
+            out["mask"] = mask
+        return out
+
+
+@dataclass
+class GroupedMoESpec:
+    """Softmax-routed mixture: ``experts`` squared-ReLU experts of width ``ff`` plus ``identity`` identity experts, ``top``
+    of them per token, chosen inside the ``keep_groups`` best of ``groups`` equal groups; an optional shared expert of
+    width ``shared_ff`` for every token."""
+
+    experts: int
+    identity: int
+    top: int
+    groups: int
+    keep_groups: int
+    ff: int
+    shared_ff: int = 0
+    kind = "moe"
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "GroupedMoESpec":
+        if d.get("kind", "moe") != "moe":
+            raise ValueError(f"unknown feed-forward kind {d.get('kind')!r}")
+        r = d["router"]
+        gr = r.get("groups") or {}
+        out = cls(experts=int(r["experts"]), identity=int(r.get("identity", 0) or 0), top=int(r["top"]),
+                  groups=int(gr.get("count", 1)), keep_groups=int(gr.get("keep", gr.get("count", 1))),
+                  ff=int(d["expert"]["ff"]), shared_ff=int((d.get("shared") or {}).get("ff", 0)))
+        total = out.experts + out.identity
+        if out.groups < 1 or total % out.groups or not 1 <= out.keep_groups <= out.groups:
+            raise ValueError(f"router: {total} experts do not form {out.groups} equal groups of which {out.keep_groups} are kept")
+        if not 1 <= out.top <= out.keep_groups * (total // out.groups):
+            raise ValueError(f"router: top {out.top} does not fit the kept groups")
+        return out
+
+    def to_dict(self) -> Dict[str, Any]:
+        router: Dict[str, Any] = {"experts": self.experts, "top": self.top}
+        if self.identity:
+            router["identity"] = self.identity
+        if self.groups > 1:
+            router["groups"] = {"count": self.groups, "keep": self.keep_groups}
+        out: Dict[str, Any] = {"kind": "moe", "expert": {"ff": self.ff}, "router": router}
+        if self.shared_ff:
+            out["shared"] = {"ff": self.shared_ff}
+        return out
+
+
+class ZifisunConfig:
+    """Zifisun decoder: ``config.json`` with ``architecture: "Zifisun"``, ``vocab``, ``width``, ``norm.eps``, ``streams``
+    (residual streams of the hyper-connections; absent: one plain residual), ``loop`` (``{start, stop, times}``: layers
+    ``start .. stop - 1`` run ``times`` times in a row with the same weights; absent: every layer once) and a ``layers``
+    list of ``{type, mixer, mlp}`` entries; ``type`` is ``latent_attention`` or ``attention``, ``mlp`` null or a
+    ``GroupedMoESpec`` entry."""
+
+    model_type = "zifisun"
+    architecture = "Zifisun"
+    MIXERS = {"latent_attention": RotaryLatentSpec, "attention": NormedAttentionSpec}
+
+    def __init__(self, vocab_size: int, hidden_size: int, layers, norm_eps: float = 1e-6, streams: int = 0,
+                 loop_start: int = 0, loop_stop: int = 0, loop_times: int = 1, pad_token_id: int = -1,
+                 eos_token_id: Optional[int] = None):
+        self.vocab_size = int(vocab_size)
+        self.hidden_size = int(hidden_size)
+        self.layers = list(layers)
+        self.norm_eps = float(norm_eps)
+        self.streams = int(streams or 0)  # 0: no hyper-connection tensors, a plain residual
+        self.loop_start, self.loop_stop, self.loop_times = int(loop_start), int(loop_stop), int(loop_times)
+        self.pad_token_id = pad_token_id
+        self.eos_token_id = eos_token_id
+        if not 0 <= self.loop_start <= self.loop_stop <= len(self.layers) or self.loop_times < 1:
+            raise ValueError(f"loop {self.loop_start}..{self.loop_stop} x {self.loop_times} does not fit "
+                             f"{len(self.layers)} layers")
+
+    def layer_runs(self) -> list:
+        """The layer index of every layer run, in order (a looped layer appears once per pass; each run has its own
+        cache)."""
+        a, b = self.loop_start, self.loop_stop
+        return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, len(self.layers)))
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layer_runs())
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "ZifisunConfig":
+        layers = []
+        for i, e in enumerate(d["layers"]):
+            if e["type"] not in cls.MIXERS:
+                raise ValueError(f"layer {i}: Zifisun has no mixer {e['type']!r}")
+            f = e.get("mlp")
+            layers.append(LayerSpec(cls.MIXERS[e["type"]].from_dict(e["mixer"]),
+                                    GroupedMoESpec.from_dict(f) if f is not None else None))
+        loop = d.get("loop") or {}
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], layers=layers, norm_eps=d["norm"]["eps"],
+                   streams=d.get("streams", 0), loop_start=loop.get("start", 0), loop_stop=loop.get("stop", 0),
+                   loop_times=loop.get("times", 1), pad_token_id=d.get("pad_token_id", -1),
+                   eos_token_id=d.get("eos_token_id"))
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+                               "norm": {"eps": self.norm_eps},
+                               "layers": [{"type": ls.mixer.type, "mixer": ls.mixer.to_dict(),
+                                           "mlp": ls.mlp.to_dict() if ls.mlp is not None else None} for ls in self.layers]}
+        if self.streams:
+            out["streams"] = self.streams
+        if self.loop_stop > self.loop_start and self.loop_times != 1:
+            out["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        return out
+
+    def save_pretrained(self, save_directory: str) -> None:
+        os.makedirs(save_directory, exist_ok=True)
+        with open(os.path.join(save_directory, "config.json"), "w") as f:
+            json.dump(self.to_dict(), f, indent=1, sort_keys=True)
+
+    @classmethod
+    def from_pretrained(cls, path: str) -> "ZifisunConfig":
+        if os.path.isdir(path):
+            path = os.path.join(path, "config.json")
+        with open(path) as f:
+            return cls.from_dict(json.load(f))
+
+    def __eq__(self, other: object) -> bool:
+        return isinstance(other, ZifisunConfig) and self.to_dict() == other.to_dict()
+
+    def __repr__(self) -> str:
+        return f"ZifisunConfig {json.dumps(self.to_dict(), sort_keys=True)}"

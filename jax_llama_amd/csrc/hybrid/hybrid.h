@@ -12,10 +12,10 @@
 
 namespace jla {
 
-// out[M, D] (fp32) = table[ids[m], col0 : col0 + D] * scale; table rows are `ld` elements apart. Ids outside [0, V)
-// read row 0.
+// out[c][M, D] (fp32) = table[ids[m], col0 : col0 + D] * scale for c < copies (the same rows `copies` times: the residual
+// streams of a hyper-connected stack); table rows are `ld` elements apart. Ids outside [0, V) read row 0.
 int hy_embed_rows(const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0, float scale, float* out,
-                  int M, int D, hipStream_t s);
+                  int M, int D, int copies, hipStream_t s);
 
 // Epilogue of a row linear. Plain forms take one accumulator, gated forms two (gate rows [0, N), up rows [N, 2N)).
 enum RowAct {
@@ -76,6 +76,37 @@ bool hy_linear_rows_is_gemv(const RowLinear& p);
 int hy_route_topk(const float* z, int ldz, int M, int top, int E, int32_t* row_expert, int32_t* row_tok, float* row_w,
                   int32_t* sort_tok, int32_t* sort_dst, float* sort_w, int32_t* offs, hipStream_t s);
 
+// Grouped softmax routing: scores = softmax(z[m, 0 : E]); the choice is made on score + correction[e] (correction
+// optional); the E experts form `groups` equal groups of neighbours, a group's score is its largest choice score, and
+// only experts of the `keep` best groups can be chosen; the `top` largest are taken (ties to the lower index
+// everywhere), weight = the chosen expert's score (not renormalised). Same outputs as hy_route_topk. E <= 1024,
+// E % groups == 0, groups <= 64, top <= keep * (E / groups).
+int hy_route_grouped(const float* z, int ldz, const float* correction, int M, int top, int E, int groups, int keep,
+                     int32_t* row_expert, int32_t* row_tok, float* row_w, int32_t* sort_tok, int32_t* sort_dst,
+                     float* sort_w, int32_t* offs, hipStream_t s);
+
+// Hyper-connections: S residual streams xs[S][M, D] (fp32). With mix != nullptr the streams are replaced in place, all
+// at once from the old ones:   xs[t][m] <- sum_s mix[s * S + t] xs[s][m] + out_w[t] * v[m],
+//   v[m] = sum_{c < nsum} w_c y[m * nsum + c] (+ extra[m]),  w_c = row_w ? row_w[m * nsum + c] : 1;
+// with row_expert, a row whose expert is >= n_real is an identity expert: it adds w_c * ident[m] and its y row is not read.
+// With next_in != nullptr: u[m] = sum_t next_in[t] xs[t][m] of the (new) streams. mix == nullptr: only u. S <= 8.
+struct HyperUpdate {
+  float* xs;
+  int S, M, D;
+  const float* mix;    // [S, S] indexed [from, to]
+  const float* out_w;  // [S]
+  const float* y;      // [M * nsum, D]
+  int nsum;
+  const float* row_w;        // optional [M * nsum]
+  const int32_t* row_expert; // optional [M * nsum]
+  int n_real;
+  const float* ident;  // [M, D], with row_expert
+  const float* extra;  // optional [M, D]
+  const float* next_in;  // optional [S]
+  float* u;              // [M, D], with next_in
+};
+int hy_hc_update(const HyperUpdate& p, hipStream_t s);
+
 // x[m, :] += (sum_{c < nsum} y[m * nsum + c, :]) * ysc / sqrt(mean(.^2) + eps) * w   (w: one number, or D numbers).
 // x == nullptr: out-of-place into `out` without the add (a plain RMS norm).
 // extra (optional, [M, D]): sigmoid(extra_gate[m * ldg]) * extra[m, :] joins the sum before the norm (extra_gate ==
@@ -108,6 +139,9 @@ struct AttnPrep {
   float eps;
   float temp_coef;  // 0: no query temperature
   int temp_every;
+  const float* q_w;  // optional [dim]: gain of the q norm (shared by all heads)
+  const float* k_w;  // optional [dim]: gain of the k norm
+  int norm_v;        // 0: values are cached as projected
 };
 // Per head: q, k divided by their RMS over dim (v over vdim); q times 1 + coef * ln(floor((p + 1) / every) + 1);
 // k, v written to the cache at slot + s.
@@ -122,8 +156,15 @@ struct LatentPrep {
   void* cache;        // [B, 1, T, rank]
   int cbf16;
   float eps;
-  float* q;           // optional [M, q_cols]: dense copy of proj's columns [0, q_cols) (the queries of the same fused
-  int q_cols;         // projection), for the per-head linear that follows
+  float* q;           // optional [M, q_cols]: dense copy of proj's columns [q_col0, q_col0 + q_cols) (the queries of the
+  int q_cols;         // same fused projection), for the linear that follows
+  int q_col0;
+  const float* q_norm_w;  // optional [q_cols]: the copy is RMS-normed with this plain gain (a query latent)
+  int row;                // width of a cache row, >= rank: the columns behind the latent, proj[col0 + rank, col0 + row), are
+                          // cached as they are behind it, their first 2 rot_half numbers rotated by the token's position
+  const double* rot_freq; // optional [rot_half]: pair (2i, 2i + 1) turns by position * rot_freq[i]
+  int rot_half;
+  const int32_t* positions;  // [M], with rot_freq
 };
 // cache[b, 0, slot + s, :] = proj_latent / sqrt(mean(.^2) + eps) * w: the one vector per token that latent attention
 // keeps (keys and values of every head are linear maps of it).
@@ -147,6 +188,11 @@ struct AttnBias {
   void* vt_ws;  // prefill: hy_attn_prefill_ws_bytes(...) bytes for the transposed values (nullptr: the plain kernel)
   int chunk;    // > 0: query at slot i sees only keys j <= i with floor(j / chunk) == floor(i / chunk)
   const float* head_scale;  // optional [H]: head h's scores are (q . k * scale) * head_scale[h]
+  int window;      // > 0 (chunk == 0): query at slot i sees key j <= i only if i - j < window or j < keep_first
+  int keep_first;
+  const float* gate;  // optional: head h's output of token m is multiplied by sigmoid(gate[m * ldg + h])
+  int ldg;
+  int ldv;         // elements between value rows (>= vdim; the values are the first vdim numbers of each row)
 };
 int hy_attn_bias(const AttnBias& p, hipStream_t s);
 long long hy_attn_prefill_ws_bytes(int B, int S, int G, int dim, int vdim, int T, int cbf16);
@@ -223,8 +269,9 @@ int hy_rope_prep(const RopePrep& p, hipStream_t s);
 
 // out[m * ldo + h * n + d] = gain * turn(a[m * lda + h * n + .], sign * positions[m])[d]: the first 2 half numbers of
 // every head rotated (freq == nullptr: none, a scaled copy)
+// offset: the rotated numbers start there within each head; interleaved: number 2i pairs with 2i + 1 instead. out may be a.
 int hy_rotate_heads(const float* a, int lda, const int32_t* positions, const double* freq, int half, int M, int H, int n,
-                    float sign, float gain, float* out, int ldo, hipStream_t s);
+                    float sign, float gain, float* out, int ldo, int offset, int interleaved, hipStream_t s);
 
 // out[i][m][:] = h[m] + (h[m - 1] - h[m]) * mu[i] for i < n; the row before a sequence's first is prev[b] (then set to
 // the sequence's last row)

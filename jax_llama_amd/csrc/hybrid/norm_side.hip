@@ -1,6 +1,8 @@
 // Row kernels of the hybrid stack: embedding-slice gather, the norm on a sublayer's OUTPUT fused with the residual add
-// (x += rms_norm(sum of the chosen experts' outputs) * w, w one number or a vector), and the per-layer token-side gate
-// (gelu_tanh(gate projection) * a slice of a second embedding table). fp32 statistics and residual.
+// (x += rms_norm(sum of the chosen experts' outputs) * w, w one number or a vector), the per-layer token-side gate
+// (gelu_tanh(gate projection) * a slice of a second embedding table), the latent-attention prep (normed latent, normed
+// query latent, rotated shared key part, cache write) and the hyper-connection update of several residual streams.
+// fp32 statistics and residual.
 #include "hy_util.h"
 #include "hybrid.h"
 
@@ -11,22 +13,27 @@ JLA_DEV float ns_ld(const bf16_t* p) { return bf2f(*p); }
 
 template <typename WT>
 __global__ void __launch_bounds__(256) embed_rows_kernel(const int32_t* ids, const WT* table, int V, int ld, int col0,
-                                                         float scale, float* out, int D) {
-  const int m = blockIdx.x;
+                                                         float scale, float* out, int D, int copies) {
+  const int m = blockIdx.x, M = gridDim.x;
   int id = ids[m];
   id = id < 0 || id >= V ? 0 : id;
   const WT* row = table + (size_t)id * ld + col0;
-  for (int d = threadIdx.x; d < D; d += 256) out[(size_t)m * D + d] = ns_ld(row + d) * scale;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    const float v = ns_ld(row + d) * scale;
+    for (int c = 0; c < copies; ++c) out[((size_t)c * M + m) * D + d] = v;
+  }
 }
 
 int hy_embed_rows(const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0, float scale, float* out,
-                  int M, int D, hipStream_t s) {
-  if (M < 0 || D < 1 || V < 1 || col0 < 0 || col0 + D > ld) return -1;
+                  int M, int D, int copies, hipStream_t s) {
+  if (M < 0 || D < 1 || V < 1 || col0 < 0 || col0 + D > ld || copies < 1) return -1;
   if (M == 0) return 0;
   if (wbf16)
-    embed_rows_kernel<bf16_t><<<M, 256, 0, s>>>(ids, reinterpret_cast<const bf16_t*>(table), V, ld, col0, scale, out, D);
+    embed_rows_kernel<bf16_t><<<M, 256, 0, s>>>(ids, reinterpret_cast<const bf16_t*>(table), V, ld, col0, scale, out, D,
+                                                copies);
   else
-    embed_rows_kernel<float><<<M, 256, 0, s>>>(ids, reinterpret_cast<const float*>(table), V, ld, col0, scale, out, D);
+    embed_rows_kernel<float><<<M, 256, 0, s>>>(ids, reinterpret_cast<const float*>(table), V, ld, col0, scale, out, D,
+                                               copies);
   JLA_CHECK_LAUNCH();
   return 0;
 }
@@ -172,6 +179,15 @@ int hy_gelu_gate_rows(const float* gp, const int32_t* ids, const void* table, in
   return 0;
 }
 
+JLA_DEV void lp_st(float* p, float v) { *p = v; }
+JLA_DEV void lp_st(bf16_t* p, float v) { *p = f2bf(v); }
+// sine and cosine of position * freq, the angle formed and reduced to [-pi, pi] in 64-bit
+JLA_DEV void lp_sincos(int pos, double freq, float* s, float* c) {
+  const double a = (double)pos * freq;
+  const double r = a - 6.283185307179586476925 * rint(a * 0.159154943091895335769);
+  sincosf((float)r, s, c);
+}
+
 // one workgroup per token: RMS norm of the down-projected latent with its gain, written to the cache row of slot + s,
 // and the dense copy of the queries (four loads in flight per thread: a decode step is one token, so the copy's
 // latency, not its bandwidth, is what shows)
@@ -180,15 +196,33 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(LatentPrep p) {
   __shared__ float red[16];
   const int tid = threadIdx.x, m = blockIdx.x;
   if (p.q) {
-    const float* src = p.proj + (size_t)m * p.ld;
+    const float* src = p.proj + (size_t)m * p.ld + p.q_col0;
     float* dst = p.q + (size_t)m * p.q_cols;
-    for (int d0 = 0; d0 < p.q_cols; d0 += 1024) {
-      float v[4];
+    float qsc = 1.f;
+    if (p.q_norm_w) {  // a query latent: RMS over the copied columns
+      float qs = 0.f;
+      for (int d0 = 0; d0 < p.q_cols; d0 += 1024) {
+        float v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = src[min(d0 + tid + 256 * u, p.q_cols - 1)];
+        for (int u = 0; u < 4; ++u) v[u] = src[min(d0 + tid + 256 * u, p.q_cols - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (d0 + tid + 256 * u < p.q_cols) qs = fmaf(v[u], v[u], qs);
+      }
+      qs = block_sum(qs, red);
+      qsc = 1.f / sqrtf(qs / (float)p.q_cols + p.eps);
+    }
+    for (int d0 = 0; d0 < p.q_cols; d0 += 1024) {
+      float v[4], g[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int d = min(d0 + tid + 256 * u, p.q_cols - 1);
+        v[u] = src[d];
+        g[u] = p.q_norm_w ? p.q_norm_w[d] : 1.f;
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        if (d0 + tid + 256 * u < p.q_cols) dst[d0 + tid + 256 * u] = v[u];
+        if (d0 + tid + 256 * u < p.q_cols) dst[d0 + tid + 256 * u] = p.q_norm_w ? v[u] * qsc * g[u] : v[u];
     }
   }
   const float* row = p.proj + (size_t)m * p.ld + p.col0;
@@ -212,7 +246,21 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(LatentPrep p) {
   const float sc = 1.f / sqrtf(ss / (float)p.rank + p.eps);
   const int b = m / p.S, t = *p.slot + (m - b * p.S);
   if (t < 0 || t >= p.T) return;  // cache full: the write is dropped
-  CT* dst = reinterpret_cast<CT*>(p.cache) + ((size_t)b * p.T + t) * p.rank;
+  CT* dst = reinterpret_cast<CT*>(p.cache) + ((size_t)b * p.T + t) * p.row;
+  // behind the latent: the shared key part, rotated in pairs (2i, 2i + 1) by the token's position
+  const int tail = p.row - p.rank;
+  if (tail > 0) {
+    const float* tr = row + p.rank;
+    const int pos = p.rot_freq ? p.positions[m] : 0;
+    for (int i = tid; i < p.rot_half; i += 256) {
+      float sn, cs;
+      lp_sincos(pos, p.rot_freq[i], &sn, &cs);
+      const float a = tr[2 * i], c = tr[2 * i + 1];
+      lp_st(dst + p.rank + 2 * i, a * cs - c * sn);
+      lp_st(dst + p.rank + 2 * i + 1, c * cs + a * sn);
+    }
+    for (int d = 2 * p.rot_half + tid; d < tail; d += 256) lp_st(dst + p.rank + d, tr[d]);
+  }
   if (p.rank <= 256 * LP_REGS) {
 #pragma unroll
     for (int u = 0; u < LP_REGS; ++u) {
@@ -233,13 +281,88 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(LatentPrep p) {
 }
 
 int hy_latent_prep(const LatentPrep& p, hipStream_t s) {
-  if (p.B < 0 || p.S < 1 || p.rank < 1 || p.T < 1 || p.col0 < 0 || p.col0 + p.rank > p.ld) return -1;
-  if (p.q && (p.q_cols < 1 || p.q_cols > p.ld)) return -2;
+  if (p.B < 0 || p.S < 1 || p.rank < 1 || p.T < 1 || p.col0 < 0 || p.row < p.rank || p.col0 + p.row > p.ld) return -1;
+  if (p.q && (p.q_cols < 1 || p.q_col0 < 0 || p.q_col0 + p.q_cols > p.ld)) return -2;
+  if (p.q_norm_w && !p.q) return -2;
+  if (p.rot_half < 0 || 2 * p.rot_half > p.row - p.rank || (p.rot_half > 0 && (!p.rot_freq || !p.positions))) return -4;
   const long long M = (long long)p.B * p.S;
   if (M == 0) return 0;
   if (M > 0x7fffffff) return -3;
   if (p.cbf16) latent_prep_kernel<bf16_t><<<(unsigned)M, 256, 0, s>>>(p);
   else latent_prep_kernel<float><<<(unsigned)M, 256, 0, s>>>(p);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+// one workgroup per token, a thread per column (in steps of 256): every stream's old value of the column is read before
+// any is written, so the replacement is in place
+template <int S>
+__global__ void __launch_bounds__(256) hc_update_kernel(HyperUpdate p) {
+  const int m = blockIdx.x;
+  float mixv[S][S], outw[S], inw[S];
+#pragma unroll
+  for (int a = 0; a < S; ++a) {
+    outw[a] = p.mix ? p.out_w[a] : 0.f;
+    inw[a] = p.next_in ? p.next_in[a] : 0.f;
+#pragma unroll
+    for (int t = 0; t < S; ++t) mixv[a][t] = p.mix ? p.mix[a * S + t] : (a == t ? 1.f : 0.f);
+  }
+  // the weights of this token's rows; identity experts pool into one weight on `ident`
+  constexpr int MAXC = 16;
+  float wc[MAXC], wid = 0.f;
+  const int nsum = p.mix ? p.nsum : 0;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    wc[c] = 0.f;
+    if (c < nsum) {
+      const size_t r = (size_t)m * nsum + c;
+      const float w = p.row_w ? p.row_w[r] : 1.f;
+      const bool real = !p.row_expert || p.row_expert[r] < p.n_real;
+      wc[c] = real ? w : 0.f;
+      wid += real ? 0.f : w;
+    }
+  }
+  const size_t plane = (size_t)p.M * p.D;
+  for (int d = threadIdx.x; d < p.D; d += 256) {
+    const size_t at = (size_t)m * p.D + d;
+    float xv[S];
+#pragma unroll
+    for (int a = 0; a < S; ++a) xv[a] = p.xs[a * plane + at];
+    float v = 0.f;
+    if (p.mix) {
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c)
+        if (c < nsum && wc[c] != 0.f) v = fmaf(wc[c], p.y[((size_t)m * nsum + c) * p.D + d], v);
+      if (wid != 0.f) v = fmaf(wid, p.ident[at], v);
+      if (p.extra) v += p.extra[at];
+    }
+    float u = 0.f;
+#pragma unroll
+    for (int t = 0; t < S; ++t) {
+      float nv = xv[t];
+      if (p.mix) {
+        nv = outw[t] * v;
+#pragma unroll
+        for (int a = 0; a < S; ++a) nv = fmaf(mixv[a][t], xv[a], nv);
+        p.xs[t * plane + at] = nv;
+      }
+      u = fmaf(inw[t], nv, u);
+    }
+    if (p.next_in) p.u[at] = u;
+  }
+}
+
+int hy_hc_update(const HyperUpdate& p, hipStream_t s) {
+  if (p.S < 1 || p.S > 8 || p.M < 0 || p.D < 1 || !p.xs) return -1;
+  if (p.mix && (!p.out_w || !p.y || p.nsum < 1 || p.nsum > 16)) return -2;
+  if (p.mix && p.row_expert && (!p.row_w || !p.ident)) return -3;
+  if ((p.next_in != nullptr) != (p.u != nullptr) || (!p.mix && !p.next_in)) return -4;
+  if (p.M == 0) return 0;
+  switch (p.S) {
+#define HC_CASE(N) case N: hc_update_kernel<N><<<p.M, 256, 0, s>>>(p); break
+    HC_CASE(1); HC_CASE(2); HC_CASE(3); HC_CASE(4); HC_CASE(5); HC_CASE(6); HC_CASE(7); HC_CASE(8);
+#undef HC_CASE
+  }
   JLA_CHECK_LAUNCH();
   return 0;
 }

@@ -45,6 +45,7 @@ class LayerListLM:
         self.embed_scale = 1.0
         self.embed_norm: Optional[torch.Tensor] = None  # fp32 [D]: gain of an RMS norm on the embedding
         self.logit_softcap = 0.0                        # logits <- cap * tanh(logits / cap) when > 0
+        self.streams = 0  # > 0: the blocks work on that many residual streams [S, M, D] (hyper-connections)
         self.final_norm: Optional[torch.Tensor] = None  # fp32 gain of the last norm: one number or [D]
         self.head: Optional[torch.Tensor] = None
         if _do_init:
@@ -125,14 +126,25 @@ class LayerListLM:
         d = self.config.hidden_size
         idf = ids.reshape(-1).to(self.device, torch.int32).contiguous()
         ctx = StepContext(idf, positions.reshape(-1).to(self.device, torch.int32).contiguous(), b, s, cache, slot0)
-        x = hy.embed_rows(idf, self.embed, scale=self.embed_scale)
-        if self.embed_norm is not None:
-            x = hy.rms_rows(x, self.embed_norm, self.eps)
         hidden = []
-        for blk in self.blocks:
-            blk(x, ctx)
-            if collect_hidden:
-                hidden.append(x.reshape(b, s, d).clone())
+        if self.streams:
+            # every stream starts as the embedding; a block leaves the next one's input sum in ctx.u, the last block the
+            # sum of the streams: the residual that the final norm reads
+            xs = hy.embed_rows(idf, self.embed, scale=self.embed_scale, copies=self.streams).reshape(self.streams, b * s, d)
+            ones = self._stream_ones()
+            for blk in self.blocks:
+                blk(xs, ctx)
+                if collect_hidden:
+                    hidden.append(hy.hc_in(xs, ones).reshape(b, s, d))
+            x = ctx.u if ctx.u is not None else hy.hc_in(xs, ones)
+        else:
+            x = hy.embed_rows(idf, self.embed, scale=self.embed_scale)
+            if self.embed_norm is not None:
+                x = hy.rms_rows(x, self.embed_norm, self.eps)
+            for blk in self.blocks:
+                blk(x, ctx)
+                if collect_hidden:
+                    hidden.append(x.reshape(b, s, d).clone())
         if logits_mode == "none":
             return None, x, hidden, []
         if logits_mode in ("last", "argmax"):
@@ -147,6 +159,12 @@ class LayerListLM:
         logits = hy.linear(hy.rms_rows(xl, self.final_norm, self.eps), self.head,
                            act=hy.ACT_SOFTCAP if cap > 0 else hy.ACT_NONE, limit=cap)
         return logits, x, hidden, []
+
+    def _stream_ones(self) -> torch.Tensor:
+        ones = getattr(self, "_ones", None)
+        if ones is None or ones.numel() != self.streams:
+            ones = self._ones = torch.ones(self.streams, dtype=F32, device=self.device)
+        return ones
 
     def gather_logits(self, logits_local: torch.Tensor) -> torch.Tensor:
         return logits_local

@@ -24,7 +24,16 @@ the same mechanisms with other values.
   GatedDenseFF    : dense feed-forward with a two-accumulator (gated) activation.
   PreNormBlock    : ``x += sublayer(rms_norm(x))`` with the residual add in the output projection's epilogue.
 
-The blocks of the last group split a sublayer into ``features(h, ctx, out=None, gain=1.0)`` (everything up to the output
+  RotaryLatentAttention : latent attention whose queries go through a normed latent too, with one rotated key part per
+                    token shared by all heads, a sliding window and a sigmoid gate per head on the output.
+  NormedGatedAttention : attention without positions: weighted per-head RMS norm of q and k, a sliding window that may
+                    keep the sequence's first keys, a sigmoid gate per head on the output.
+  GroupedMoE      : softmax-score router with a selection bias, expert groups and identity experts; squared-ReLU experts
+                    weighted on their output; a shared expert.
+  HyperBlock      : pre-norm sublayers over several residual streams (hyper-connections): a sublayer reads a weighted
+                    sum of the streams, and its result is added to a mixed copy of them.
+
+The blocks of the group before the last split a sublayer into ``features(h, ctx, out=None, gain=1.0)`` (everything up to the output
 projection; ``out`` a column slice to write into, ``gain`` a scalar folded into the last elementwise step) and the
 matrix ``w_o``, so a block can fuse the projection with the residual add and ``SideBySide`` can run one projection for
 all of its members.
@@ -49,6 +58,7 @@ class StepContext:
     s: int
     cache: object            # HybridCache (or a row view)
     slot0: object            # int, or device int32[1] (graph-capturable)
+    u: Optional[torch.Tensor] = None  # hyper-connected stacks: the next sublayer's input sum, left by the last write
 
 
 class BiasedAttention:
@@ -419,3 +429,179 @@ class PreNormBlock:
         hy.linear_add_(x, self.mixer.features(hy.RmsInput(x, self.norm1, self.eps), ctx), self.mixer.w_o)
         if self.mlp is not None:
             hy.linear_add_(x, self.mlp.features(hy.RmsInput(x, self.norm2, self.eps), ctx), self.mlp.w_o)
+
+
+class RotaryLatentAttention(LatentAttention):
+    """Latent attention with positions. Per token the cache holds ``kv_rank`` RMS-normed numbers (from which every head's
+    plain keys and its values are linear maps) followed by ``rot_dim`` numbers rotated by the token's position: one
+    rotated key part shared by all heads. Queries come from a latent of their own (down projection, RMS norm with a plain
+    gain, up projection) and are laid out per head as ``dim`` plain numbers, then ``rot_dim`` rotated ones; the score is
+    ``(q_plain . k_plain + q_rot . k_rot) * scale``. Rotation pairs number ``2i`` with ``2i + 1``. ``window > 0``: a
+    query sees the last ``window`` positions (and the first ``keep_first`` of the sequence). Each head's output is
+    multiplied by the sigmoid of one more projection of the mixer's input.
+
+    Both forms of ``LatentAttention`` carry over with the rotated part as ``rot_dim`` more key numbers: in the latent
+    space a head's query becomes ``[W_uk[h]^T q_plain | q_rot]`` against the cache row itself (the values are the row's
+    first ``kv_rank`` numbers); expanded, a head's key is ``[W_uk[h] c | k_rot]``. The maps are stored with an identity
+    block for the rotated part, so both run as the same per-head linears."""
+
+    def __init__(self, layer_idx: int, spec, eps: float, w_in: torch.Tensor, dq_norm: torch.Tensor, w_uq: torch.Tensor,
+                 dkv_norm: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, freq: Optional[torch.Tensor],
+                 w_o: torch.Tensor):
+        self.i = layer_idx
+        self.spec = spec
+        self.eps = eps
+        self.w_in = w_in          # [q_rank + kv_rank + rot_dim + H, D]: query latent, key / value latent, rotated key, gates
+        self.dq_norm, self.dkv_norm = dq_norm, dkv_norm  # fp32 [q_rank], [kv_rank]
+        self.w_uq = w_uq          # [H (dim + rot_dim), q_rank]
+        self.freq = freq          # float64 [rot_dims / 2] or None
+        self.w_o = w_o            # [D, H vdim]
+        nh, dim, rot, rank = spec.heads, spec.dim, spec.rot_dim, spec.kv_rank
+        eye = torch.eye(rot, dtype=w_uk.dtype, device=w_uk.device)
+        wk = torch.zeros(nh, dim + rot, rank + rot, dtype=w_uk.dtype, device=w_uk.device)
+        wk[:, :dim, :rank] = w_uk
+        wk[:, dim:, rank:] = eye
+        self.w_uk = wk                                   # [H, dim + rot, rank + rot]: a head's keys from a cache row
+        self.w_qk = wk.transpose(1, 2).contiguous()      # [H, rank + rot, dim + rot]: queries into the cache row's space
+        wv = torch.zeros(nh, spec.vdim, rank + rot, dtype=w_uv.dtype, device=w_uv.device)
+        wv[:, :, :rank] = w_uv
+        self.w_uv_row = wv        # [H, vdim, rank + rot]: a head's values from a cache row
+        self.w_uv = w_uv          # [H, vdim, rank]: ... from the attended latent
+
+    def expands(self, s: int, n: int, bf16: bool) -> bool:
+        sp = self.spec
+        if s < self.EXPAND_MIN_TOKENS:
+            return False
+        seen = min(n, sp.window + sp.keep_first) if sp.window else n
+        pairs = s * min(seen, (n - s) + (s + 1) / 2.0)
+        row, kd = sp.kv_rank + sp.rot_dim, sp.dim + sp.rot_dim
+        mma = bf16 and kd in self.MMA_SIZES and sp.vdim in self.MMA_SIZES
+        # (in the latent space keys and values differ in width: always the plain kernels)
+        latent = s * row * (kd + sp.vdim) + pairs * (row + sp.kv_rank) * self.PLAIN_KERNEL_COST
+        expanded = min(n, s + seen) * row * (kd + sp.vdim) + pairs * (kd + sp.vdim) * (1.0 if mma else self.PLAIN_KERNEL_COST)
+        return expanded < latent
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        sp = self.spec
+        m, nh, rank, rot = ctx.b * ctx.s, sp.heads, sp.kv_rank, sp.rot_dim
+        kd, row = sp.dim + rot, rank + rot
+        proj = hy.linear(h, self.w_in)
+        c, _ = ctx.cache.layer(self.i)
+        cq = hy.latent_rope_prep(proj, 0, self.dq_norm, sp.q_rank, self.dkv_norm, self.freq, ctx.positions, ctx.slot0,
+                                 ctx.b, ctx.s, c, self.eps)
+        q = hy.linear(cq, self.w_uq)
+        if self.freq is not None:
+            hy.rotate_heads(q, ctx.positions, self.freq, nh, out=q, offset=sp.dim, interleaved=True)
+        gate = proj[:, sp.q_rank + row:sp.q_rank + row + nh]
+        s0 = ctx.cache.index if torch.is_tensor(ctx.slot0) else int(ctx.slot0)  # (host mirror of the slot)
+        n = s0 + ctx.s
+        wide = row > hy.ATTN_MAX_HEAD
+        if wide and c.is_cuda and torch.cuda.is_current_stream_capturing():
+            raise NotImplementedError(f"latent attention: a cache row of {row} > {hy.ATTN_MAX_HEAD} in a captured step")
+        if wide or (ctx.s > 1 and self.expands(ctx.s, n, c.dtype == torch.bfloat16)):
+            # only the keys some query of the step can see are expanded: with a window and no kept first keys, the
+            # scratch keys start at `first` and the step's slot is counted from there
+            first = max(0, s0 - sp.window + 1) // 64 * 64 if sp.window and not sp.keep_first else 0
+            k = hy.latent_expand(c, n, self.w_uk, first)
+            v = hy.latent_expand(c, n, self.w_uv_row, first)
+            o = hy.attn_bias(q.reshape(ctx.b, ctx.s, nh, kd), k, v, ctx.slot0 if first == 0 else s0 - first, sp.scale,
+                             window=sp.window, keep_first=sp.keep_first, gate=gate)
+            return hy.linear(o, self.w_o)
+        ql = hy.heads_linear(q.reshape(m, nh, kd), self.w_qk)
+        a = hy.attn_bias(ql.reshape(ctx.b, ctx.s, nh, row), c, c, ctx.slot0, sp.scale, window=sp.window,
+                         keep_first=sp.keep_first, gate=gate, vdim=rank)
+        o = hy.heads_linear(a.reshape(m, nh, rank), self.w_uv)
+        return hy.linear(o.reshape(m, nh * sp.vdim), self.w_o)
+
+
+class NormedGatedAttention:
+    """Softmax attention over this layer's own keys and values, without positions: every q / k head is divided by its
+    root mean square and multiplied by a gain vector shared by all heads (``q_norm`` / ``k_norm [dim]``), values are
+    cached as projected; ``window > 0``: a query sees the last ``window`` positions and the first ``keep_first`` of the
+    sequence; each head's output is multiplied by the sigmoid of one more projection of the mixer's input."""
+
+    def __init__(self, layer_idx: int, spec, eps: float, w_in: torch.Tensor, q_norm: Optional[torch.Tensor],
+                 k_norm: Optional[torch.Tensor], gated: bool, w_o: torch.Tensor):
+        self.i = layer_idx
+        self.spec = spec
+        self.eps = eps
+        self.w_in = w_in  # [H dim + G dim + G vdim (+ H), D]: q | k | v | gates
+        self.q_norm, self.k_norm, self.gated = q_norm, k_norm, gated
+        self.w_o = w_o    # [D, H vdim]
+
+    def __call__(self, h, ctx: StepContext) -> torch.Tensor:
+        sp = self.spec
+        proj = hy.linear(h, self.w_in)
+        cols = (sp.heads + sp.kv_heads) * sp.dim + sp.kv_heads * sp.vdim
+        kc, vc = ctx.cache.layer(self.i)
+        q = hy.attn_prep(proj[:, :cols], ctx.positions, ctx.slot0, ctx.b, ctx.s, sp.heads, sp.kv_heads, sp.dim, sp.vdim,
+                         kc, vc, self.eps, q_w=self.q_norm, k_w=self.k_norm, norm_v=False)
+        gate = proj[:, cols:cols + sp.heads] if self.gated else None
+        a = hy.attn_bias(q, kc, vc, ctx.slot0, sp.scale, window=sp.window, keep_first=sp.keep_first, gate=gate)
+        return hy.linear(a, self.w_o)
+
+
+@dataclass
+class MixtureOut:
+    """A mixture's result before it is summed: ``y [M * nsum, D]`` with a weight and an expert per row (rows of experts
+    ``>= n_real`` stand for identity experts: the weight times ``ident [M, D]``), plus a per-token summand ``extra``."""
+
+    y: torch.Tensor
+    nsum: int
+    row_w: torch.Tensor
+    row_expert: torch.Tensor
+    n_real: int
+    ident: torch.Tensor
+    extra: Optional[torch.Tensor] = None
+
+
+class GroupedMoE:
+    """Mixture of one-accumulator experts (``W_down relu(W_up h)^2``) chosen by a softmax-score router: logits over the
+    real experts and ``identity`` identity experts behind them (an identity expert returns its input), scores = softmax,
+    the choice made on score + ``correction`` within the ``keep`` best of ``groups`` equal groups, the ``top`` largest
+    chosen, each weighted on its OUTPUT by its score (not renormalised). An optional shared expert of the same form runs
+    for every token. The router is an fp32 matrix in both number formats."""
+
+    def __init__(self, experts: int, identity: int, top: int, groups: int, keep: int, w_router: torch.Tensor,
+                 correction: Optional[torch.Tensor], w_up: Optional[torch.Tensor], w_down: Optional[torch.Tensor],
+                 shared_up: Optional[torch.Tensor] = None, shared_down: Optional[torch.Tensor] = None,
+                 act: int = hy.ACT_RELU2):
+        self.experts, self.identity, self.top, self.groups, self.keep = experts, identity, top, groups, keep
+        self.w_router = w_router      # fp32 [E + I, D]
+        self.correction = correction  # fp32 [E + I] or None
+        self.w_up, self.w_down = w_up, w_down  # [E, ff, D], [E, D, ff]
+        self.shared_up, self.shared_down, self.act = shared_up, shared_down, act
+
+    def __call__(self, h, ctx: StepContext) -> MixtureOut:
+        hv = _value(h)  # (three products and the identity experts read the normed input: written out once)
+        z = hy.linear(hv, self.w_router)
+        y, row_expert, row_w = hy.moe_grouped(hv, z, self.correction, self.top, self.groups, self.keep, self.w_up,
+                                              self.w_down, self.act)
+        extra = None
+        if self.shared_up is not None:
+            extra = hy.linear(hy.linear(hv, self.shared_up, act=self.act), self.shared_down)
+        return MixtureOut(y, self.top, row_w, row_expert, self.experts, hv, extra)
+
+
+class HyperBlock:
+    """Pre-norm sublayers over ``S`` residual streams ``xs [S, M, D]`` (hyper-connections). Sublayer ``q`` reads
+    ``u = sum_s in_q[s] xs[s]``, computes ``y = sublayer(norm_q * rms(u))``, and replaces all streams at once:
+    ``xs[t] <- sum_s mix_q[s, t] xs[s] + out_q[t] * y``. ``S = 1`` with unit weights is the plain pre-norm residual.
+    The write of a sublayer also produces the next sublayer's ``u`` (``ctx.u``; the model's last block is given ones as
+    its successor's read weights, so it leaves the sum of the streams there)."""
+
+    def __init__(self, mixer, norm1: torch.Tensor, hc1, mlp, norm2: Optional[torch.Tensor], hc2, eps: float):
+        self.mixer, self.norm1, self.hc1 = mixer, norm1, hc1  # hc: (in [S], mix [S, S], out [S]) fp32
+        self.mlp, self.norm2, self.hc2, self.eps = mlp, norm2, hc2, eps
+        self.next_in: Optional[torch.Tensor] = None  # read weights of whatever follows this block
+
+    def __call__(self, xs: torch.Tensor, ctx) -> None:
+        u = ctx.u if ctx.u is not None else hy.hc_in(xs, self.hc1[0])
+        y = self.mixer(hy.RmsInput(u, self.norm1, self.eps), ctx)
+        after = self.hc2[0] if self.mlp is not None else self.next_in
+        u = hy.hc_update_(xs, self.hc1[1], self.hc1[2], y, next_in=after)
+        if self.mlp is not None:
+            f = self.mlp(hy.RmsInput(u, self.norm2, self.eps), ctx)
+            u = hy.hc_update_(xs, self.hc2[1], self.hc2[2], f.y, f.nsum, f.row_w, f.row_expert, f.n_real, f.ident, f.extra,
+                              next_in=self.next_in)
+        ctx.u = u

@@ -37,11 +37,18 @@ def _besulix():
     return BesulixConfig, BesulixForCausalLM
 
 
+def _zifisun():
+    from ..config import ZifisunConfig
+    from .zifisun import ZifisunForCausalLM
+    return ZifisunConfig, ZifisunForCausalLM
+
+
 # architecture name (lower case) -> () -> (config class, model class)
 MODEL_REGISTRY: Dict[str, Callable[[], Tuple[type, type]]] = {"llama": _llama, "zavevik": _zavevik,
-                                                              "zasevik": _zasevik, "besulix": _besulix}
+                                                              "zasevik": _zasevik, "besulix": _besulix,
+                                                              "zifisun": _zifisun}
 # families on the layer-list step function (models/layer_list.py): both number formats, the hybrid extension
-LAYER_LIST_FAMILIES = ("zavevik", "zasevik", "besulix")
+LAYER_LIST_FAMILIES = ("zavevik", "zasevik", "besulix", "zifisun")
 
 
 def register(name: str, factory: Callable[[], Tuple[type, type]]) -> None:

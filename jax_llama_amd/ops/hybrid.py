@@ -24,7 +24,13 @@ Mechanisms (each with its constants as arguments, usable by any model of the reg
   * ``mlstm_prep`` / ``mlstm_scan`` and ``token_shift`` / ``timemix_scan``: two linear recurrences over a carried fp32
     matrix state (a stabilised exponential-gate memory with a normaliser; a per-channel-decay memory with a bonus
     for the current token), one scan kernel; ``gated_rmsnorm`` takes either's read-out;
-  * ``linear(act=ACT_SOFTCAP)`` and ``linear_add_``: ``cap * tanh(y / cap)`` epilogue; residual add in the epilogue.
+  * ``linear(act=ACT_SOFTCAP)`` and ``linear_add_``: ``cap * tanh(y / cap)`` epilogue; residual add in the epilogue;
+  * ``attn_bias(window=, keep_first=, gate=, vdim=)``: sliding-window masks that may keep a sequence's first keys, a
+    sigmoid gate per (token, head) on the output, values that are the leading columns of the key rows;
+    ``attn_prep(q_w=, k_w=, norm_v=)``: weighted per-head q / k norms; ``latent_rope_prep`` + ``rotate_heads(offset=,
+    interleaved=)``: latent attention with a normed query latent and one rotated key part shared by all heads;
+  * ``route_grouped`` / ``moe_grouped``: softmax-score router with a selection bias, expert groups and identity
+    experts; ``hc_in`` / ``hc_update_``: several residual streams mixed around every sublayer (hyper-connections).
 """
 from __future__ import annotations
 
@@ -97,15 +103,17 @@ def _round_like(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------------------------ rows
 def embed_rows(ids: torch.Tensor, table: torch.Tensor, col0: int = 0, ncols: Optional[int] = None,
-               scale: float = 1.0) -> torch.Tensor:
-    """fp32 ``[M, ncols]`` = ``table[ids, col0 : col0 + ncols] * scale``."""
+               scale: float = 1.0, copies: int = 1) -> torch.Tensor:
+    """fp32 ``[M, ncols]`` = ``table[ids, col0 : col0 + ncols] * scale``; ``copies > 1``: ``[copies, M, ncols]``, the
+    same rows ``copies`` times (the residual streams of a hyper-connected stack all start from the embedding)."""
     ncols = table.shape[1] - col0 if ncols is None else ncols
     ids = ids.reshape(-1)
     if not _gpu(table):
-        return table[ids.long(), col0:col0 + ncols].float() * torch.tensor(scale, dtype=F32)
-    out = torch.empty(ids.numel(), ncols, dtype=F32, device=table.device)
-    ext().embed_rows(ids.to(torch.int32).contiguous(), table, int(col0), out, float(scale))
-    return out
+        x = table[ids.long(), col0:col0 + ncols].float() * torch.tensor(scale, dtype=F32)
+        return x if copies == 1 else x[None].repeat(copies, 1, 1)
+    out = torch.empty(copies * ids.numel(), ncols, dtype=F32, device=table.device)
+    ext().embed_rows(ids.to(torch.int32).contiguous(), table, int(col0), out, float(scale), int(copies))
+    return out if copies == 1 else out.reshape(copies, ids.numel(), ncols)
 
 
 # Dense bf16 linears of a prompt-sized batch run on the framework's tuned MFMA GEMM (ops.linear over the fragment-
@@ -399,6 +407,116 @@ def moe_routed(x, z: torch.Tensor, top: int, w_gu: torch.Tensor, w_down: torch.T
     return y
 
 
+def route_grouped(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int = 1, keep: int = 1):
+    """Softmax-score router over logits ``z [M, E]`` (fp32): scores ``s = softmax(z)``; the choice is made on
+    ``s + correction`` (``correction [E]``, a selection bias that does not enter the weights); the experts form
+    ``groups`` equal groups of neighbours, a group's score is its largest choice score, and only experts of the ``keep``
+    best groups can be chosen (ties to the lower index everywhere); the ``top`` largest are chosen, weight ``s`` of each
+    (not renormalised). Returns ``(row_expert [R], row_w [R])`` in (token, choice) order."""
+    zz = z.float()
+    m, e_n = zz.shape
+    sc = torch.softmax(zz, -1)
+    ch = sc + correction.float().reshape(1, -1) if correction is not None else sc.clone()
+    if groups > 1:
+        per = e_n // groups
+        gs = ch.reshape(m, groups, per).max(-1).values
+        best = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        allowed = torch.zeros(m, groups, dtype=torch.bool).scatter_(1, best, True)
+        ch = ch.masked_fill(~allowed.repeat_interleave(per, 1), float("-inf"))
+    order = torch.sort(ch, dim=-1, descending=True, stable=True).indices[:, :top]
+    return order.reshape(-1), torch.gather(sc, 1, order).reshape(-1)
+
+
+def moe_grouped(x: torch.Tensor, z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int,
+                w_up: torch.Tensor, w_down: torch.Tensor, act: int = ACT_RELU2):
+    """Experts of a ``route_grouped`` mixture: ``z [M, E + I]`` holds the logits of the ``E = w_up.shape[0]`` real
+    experts and of ``I`` identity experts behind them (an identity expert returns its input; it has no weights and runs
+    no product). ``w_up [E, F, K]``, ``w_down [E, D, F]``, one-accumulator activation ``act``. Returns
+    ``(y [M * top, D], row_expert [M * top], row_w [M * top])`` in (token, choice) order: ``y`` rows of real experts hold
+    ``W_down act(W_up x)`` unweighted, rows whose expert is ``>= E`` hold nothing (the caller's ``hc_update_`` puts the
+    weighted sum together)."""
+    m, e_n, e_all = x.shape[0], w_up.shape[0], z.shape[1]
+    r = m * top
+    if act_gated(act):
+        raise ValueError("moe_grouped: one-accumulator activations only")
+    if not _gpu(x):
+        ex, wt = route_grouped(z, correction, top, groups, keep)
+        xr = _round_like(x.float(), w_up).repeat_interleave(top, 0)
+        y = torch.zeros(r, w_down.shape[1], dtype=F32)
+        for e in ex.unique().tolist():
+            if e >= e_n:
+                continue
+            sel = (ex == e).nonzero().squeeze(1)
+            hid = _act_cpu(xr[sel] @ w_up[e].float().t(), act, 0.0, 1.0)
+            y[sel] = _round_like(hid, w_down) @ w_down[e].float().t()
+        return y, ex.to(torch.int32), wt
+    dev = x.device
+    e = ext()
+    idx = torch.empty(4 * r + e_all + 1, dtype=torch.int32, device=dev)
+    row_expert, row_tok, sort_tok, sort_dst, offs = idx[:r], idx[r:2 * r], idx[2 * r:3 * r], idx[3 * r:4 * r], idx[4 * r:]
+    wts = torch.empty(2 * r, dtype=F32, device=dev)
+    row_w, sort_w = wts[:r], wts[r:]
+    y = torch.empty(r, w_down.shape[1], dtype=F32, device=dev)
+    f = w_up.shape[1]
+    if r <= e.GEMV_MAX_R:  # decode: one GEMV per (token, choice) row; rows of identity experts are skipped on the device
+        e.route_grouped(z, correction, e_all, top, groups, keep, row_expert, row_tok, row_w, None, None, None, None)
+        h = torch.empty(r, f, dtype=F32, device=dev)
+        e.linear_rows(x, row_tok, w_up, h, None, None, row_expert, r, int(act), 0.0, 1.0, None, None, 0.0)
+        e.linear_rows(h, None, w_down, y, None, None, row_expert, r, ACT_NONE, 0.0, 1.0, None, None, 0.0)
+    else:
+        # expert-grouped over the sorted rows; identity experts sort behind the real ones, past the last offset the
+        # linears look at
+        e.route_grouped(z, correction, e_all, top, groups, keep, row_expert, row_tok, row_w, sort_tok, sort_dst, sort_w, offs)
+        keep_bf16 = w_up.dtype == BF16 and r > GROUPED_GEMV_MAX_R
+        h = torch.empty(r, f, dtype=BF16 if keep_bf16 else F32, device=dev)
+        e.linear_rows(x, sort_tok, w_up, h, None, offs, None, r, int(act), 0.0, 1.0, None, None, 0.0)
+        e.linear_rows(h, None, w_down, y, sort_dst, offs, None, r, ACT_NONE, 0.0, 1.0, None, None, 0.0)
+    return y, row_expert, row_w
+
+
+def hc_in(xs: torch.Tensor, a: torch.Tensor) -> torch.Tensor:
+    """What a sublayer of a hyper-connected stack reads: ``u [M, D] = sum_s a[s] xs[s]`` for the residual streams
+    ``xs [S, M, D]`` (fp32) and the read weights ``a [S]`` (fp32)."""
+    if not _gpu(xs):
+        return torch.einsum("s,smd->md", a.float(), xs.float())
+    u = torch.empty(xs.shape[1], xs.shape[2], dtype=F32, device=xs.device)
+    ext().hc_update(xs, None, None, None, 1, None, None, 0, None, None, a, u)
+    return u
+
+
+def hc_update_(xs: torch.Tensor, mix: torch.Tensor, out_w: torch.Tensor, y: torch.Tensor, nsum: int = 1,
+               row_w: Optional[torch.Tensor] = None, row_expert: Optional[torch.Tensor] = None, n_real: int = 0,
+               ident: Optional[torch.Tensor] = None, extra: Optional[torch.Tensor] = None,
+               next_in: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """A sublayer's write into the residual streams ``xs [S, M, D]`` (fp32, in place), all streams at once from the old
+    ones: ``xs[t] <- sum_s mix[s, t] xs[s] + out_w[t] * v`` with the sublayer's result ``v [M, D]`` put together here:
+    ``v[m] = sum_{c < nsum} w_c * y[m * nsum + c] (+ extra[m])``, ``w_c = row_w[m * nsum + c]`` (absent: 1); a row whose
+    ``row_expert`` is ``>= n_real`` stands for an identity expert and contributes ``w_c * ident[m]`` instead (its ``y`` row
+    is not read). ``next_in [S]``: also returns ``u [M, D] = sum_t next_in[t] xs[t]`` of the NEW streams, the next
+    sublayer's input (or, with ones, the residual itself)."""
+    s_n, m, d = xs.shape
+    if not _gpu(xs):
+        v = y.float().reshape(m, nsum, d)
+        if row_w is not None:
+            wt = row_w.float().reshape(m, nsum)
+            if row_expert is not None:
+                real = row_expert.reshape(m, nsum) < n_real
+                v = (torch.where(real[..., None], v, torch.zeros_like(v)) * (wt * real)[..., None]).sum(1)
+                v = v + (wt * ~real).sum(1, keepdim=True) * ident.float()
+            else:
+                v = (v * wt[..., None]).sum(1)
+        else:
+            v = v.sum(1)
+        if extra is not None:
+            v = v + extra.float()
+        new = torch.einsum("st,smd->tmd", mix.float(), xs.float()) + out_w.float()[:, None, None] * v[None]
+        xs.copy_(new)
+        return torch.einsum("s,smd->md", next_in.float(), xs) if next_in is not None else None
+    u = torch.empty(m, d, dtype=F32, device=xs.device) if next_in is not None else None
+    ext().hc_update(xs, mix, out_w, y, int(nsum), row_w, row_expert, int(n_real), ident, extra, next_in, u)
+    return u
+
+
 def norm_residual_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float, nsum: int = 1, ysc: float = 1.0,
                    extra: Optional[torch.Tensor] = None, extra_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x += rms_norm(ysc * sum of each token's nsum rows of y [+ sigmoid(extra_gate) * extra]) * w`` in place; ``w``
@@ -476,16 +594,20 @@ def distance_bias_table(rel: torch.Tensor, bias_max: int) -> torch.Tensor:
 
 def attn_prep(proj: torch.Tensor, positions: torch.Tensor, slot, b: int, s: int, heads: int, kv_heads: int, dim: int,
               vdim: int, kc: Optional[torch.Tensor], vc: Optional[torch.Tensor], eps: float, temp_coef: float = 0.0,
-              temp_every: int = 1) -> torch.Tensor:
-    """From the fused projection ``proj [B*S, H*dim (+ G*dim + G*vdim)]``: q / k divided by their per-head RMS over
-    ``dim`` (v over ``vdim``), q scaled by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)``, k / v written into
-    the caches ``[B, G, T, .]`` at ``slot + s``. ``kc is None``: the layer reads another layer's cache (q only).
-    Returns q ``[B, S, H, dim]`` fp32."""
+              temp_every: int = 1, q_w: Optional[torch.Tensor] = None, k_w: Optional[torch.Tensor] = None,
+              norm_v: bool = True) -> torch.Tensor:
+    """From the fused projection ``proj [B*S, H*dim (+ G*dim + G*vdim) (+ more)]``: q / k divided by their per-head RMS
+    over ``dim`` (times the gain ``q_w`` / ``k_w [dim]``, shared by all heads, when given), v over ``vdim``
+    (``norm_v=False``: v as projected), q scaled by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)``, k / v
+    written into the caches ``[B, G, T, .]`` at ``slot + s``. ``kc is None``: the layer reads another layer's cache (q
+    only). Returns q ``[B, S, H, dim]`` fp32."""
     m = b * s
     if not _gpu(proj):
         s0 = _slot_int(slot)
         q = proj[:, :heads * dim].float().reshape(m, heads, dim)
         q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+        if q_w is not None:
+            q = q * q_w.float()
         if temp_coef:
             p = positions.reshape(-1).to(torch.int64)
             q = q * (1.0 + temp_coef * torch.log(torch.div(p + 1, temp_every, rounding_mode="floor").float() + 1.0)
@@ -495,13 +617,17 @@ def attn_prep(proj: torch.Tensor, positions: torch.Tensor, slot, b: int, s: int,
             v = proj[:, (heads + kv_heads) * dim:(heads + kv_heads) * dim + kv_heads * vdim].float().reshape(
                 b, s, kv_heads, vdim)
             k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
-            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+            if k_w is not None:
+                k = k * k_w.float()
+            if norm_v:
+                v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
             kc[:, :, s0:s0 + s] = k.permute(0, 2, 1, 3).to(kc.dtype)
             vc[:, :, s0:s0 + s] = v.permute(0, 2, 1, 3).to(vc.dtype)
         return q.reshape(b, s, heads, dim)
     q = torch.empty(b, s, heads, dim, dtype=F32, device=proj.device)
     ext().attn_prep(proj, positions.reshape(-1).to(torch.int32).contiguous(), _slot_tensor(slot, proj.device), b, s,
-                    heads, kv_heads, dim, vdim, kc, vc, q, float(eps), float(temp_coef), int(temp_every))
+                    heads, kv_heads, dim, vdim, kc, vc, q, float(eps), float(temp_coef), int(temp_every), q_w, k_w,
+                    bool(norm_v))
     return q
 
 
@@ -519,25 +645,59 @@ def latent_prep(proj: torch.Tensor, col0: int, w: torch.Tensor, slot, b: int, s:
         cache[:, 0, s0:s0 + s] = c.reshape(b, s, rank).to(cache.dtype)
         return proj[:, :q_cols].contiguous() if q_cols else None
     q = torch.empty(b * s, q_cols, dtype=F32, device=proj.device) if q_cols else None
-    ext().latent_prep(proj, int(col0), w, _slot_tensor(slot, proj.device), b, s, cache, float(eps), q)
+    ext().latent_prep(proj, int(col0), w, _slot_tensor(slot, proj.device), b, s, cache, float(eps), q, 0, None, None, None)
     return q
 
 
-def latent_expand(cache: torch.Tensor, n: int, w: torch.Tensor) -> torch.Tensor:
-    """Per-head linear maps of the first ``n`` cached latents: ``cache [B, 1, T, rank]``, ``w [H, N, rank]`` ->
-    ``[B, H, n, N]`` in the cache's type (the layout of a key / value cache of ``H`` heads, so the attention kernels
-    take it as one). Runs the expert-grouped row linear with the heads as its experts."""
+def latent_rope_prep(proj: torch.Tensor, q_col0: int, q_w: torch.Tensor, c_col0: int, c_w: torch.Tensor,
+                     freq: Optional[torch.Tensor], positions: torch.Tensor, slot, b: int, s: int, cache: torch.Tensor,
+                     eps: float) -> torch.Tensor:
+    """The step after the fused down projection of a latent attention whose queries go through a latent too and whose
+    keys carry one rotated part shared by all heads. From ``proj [B*S, .]``:
+      * columns ``[q_col0, q_col0 + len(q_w))``: RMS-normed, times the plain gain ``q_w`` -> returned dense (fp32), the
+        input of the queries' up projection;
+      * columns ``[c_col0, c_col0 + rank)``, ``rank = len(c_w)``: RMS-normed, times ``c_w`` -> ``cache[b, 0, slot + s, :rank]``;
+      * the next ``cache.shape[3] - rank`` columns (not normed): their first ``2 len(freq)`` numbers rotated by the
+        token's position, number ``2i`` with number ``2i + 1``, angle ``position * freq[i]`` -> ``cache[..., rank:]``."""
+    rank, q_rank = c_w.numel(), q_w.numel()
+    nrot = cache.shape[3] - rank
+    if not _gpu(proj):
+        s0 = _slot_int(slot)
+        cq = proj[:, q_col0:q_col0 + q_rank].float()
+        cq = cq * torch.rsqrt(cq.pow(2).mean(-1, keepdim=True) + eps) * q_w.float()
+        c = proj[:, c_col0:c_col0 + rank].float()
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * c_w.float()
+        cache[:, 0, s0:s0 + s, :rank] = c.reshape(b, s, rank).to(cache.dtype)
+        if nrot:
+            r = proj[:, c_col0 + rank:c_col0 + rank + nrot].float().reshape(b * s, 1, nrot)
+            if freq is not None:
+                r = _turn_pairs_cpu(r, positions.reshape(-1), freq)
+            cache[:, 0, s0:s0 + s, rank:] = r.reshape(b, s, nrot).to(cache.dtype)
+        return cq.contiguous()
+    cq = torch.empty(b * s, q_rank, dtype=F32, device=proj.device)
+    ext().latent_prep(proj, int(c_col0), c_w, _slot_tensor(slot, proj.device), b, s, cache, float(eps), cq, int(q_col0), q_w,
+                      freq, positions.reshape(-1).to(torch.int32).contiguous())
+    return cq
+
+
+def latent_expand(cache: torch.Tensor, n: int, w: torch.Tensor, first: int = 0) -> torch.Tensor:
+    """Per-head linear maps of the cached latents of slots ``[first, n)``: ``cache [B, 1, T, rank]``, ``w [H, N, rank]``
+    -> ``[B, H, n - first, N]`` in the cache's type (the layout of a key / value cache of ``H`` heads whose slot 0 is the
+    cache's slot ``first``, so the attention kernels take it as one). Runs the expert-grouped row linear with the heads as
+    its experts."""
     b, _, t, rank = cache.shape
     h, nn = w.shape[0], w.shape[1]
     if not _gpu(cache):
-        y = torch.einsum("btr,hnr->bhtn", cache[:, 0, :n].float(), w.float())
+        y = torch.einsum("btr,hnr->bhtn", cache[:, 0, first:n].float(), w.float())
         return y.to(cache.dtype)
     dev = cache.device
     if cache.dtype == F32 and w.dtype == BF16:
         raise ValueError("latent_expand: an fp32 cache needs fp32 maps")
-    out = torch.empty(b, h, n, nn, dtype=cache.dtype, device=dev)
-    a_idx, dst, offs = _expand_index(b, t, n, h, dev)
-    ext().linear_rows(cache.reshape(b * t, rank), a_idx, w, out.reshape(b * h * n, nn), dst, offs, None, b * h * n,
+    cnt = n - first
+    out = torch.empty(b, h, cnt, nn, dtype=cache.dtype, device=dev)
+    a_idx, dst, offs = _expand_index(b, t, cnt, h, dev)
+    src = cache.reshape(b * t, rank)[first:] if first else cache.reshape(b * t, rank)
+    ext().linear_rows(src, a_idx, w, out.reshape(b * h * cnt, nn), dst, offs, None, b * h * cnt,
                       ACT_NONE, 0.0, 1.0, None, None, 0.0)
     return out
 
@@ -564,21 +724,28 @@ def _expand_index(b: int, t: int, n: int, h: int, device):
 def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: float, softcap: float = 0.0,
               bias: Optional[torch.Tensor] = None, max_kv: Optional[int] = None,
               sink: Optional[torch.Tensor] = None, chunk: int = 0,
-              head_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+              head_scale: Optional[torch.Tensor] = None, window: int = 0, keep_first: int = 0,
+              gate: Optional[torch.Tensor] = None, vdim: Optional[int] = None) -> torch.Tensor:
     """Causal attention of ``q [B, S, H, dim]`` (queries at cache slots ``slot + s``) over ``[B, G, T, .]`` caches:
     ``score = q.k * scale``; ``softcap * tanh(score / softcap)`` if ``softcap > 0``; ``+ bias[min(i - j, last), h]``;
     softmax over ``j <= i``, with ``exp(sink[h])`` added to the denominator when ``sink [H]`` is given (a slot without
     key or value). ``chunk > 0``: query ``i`` only sees the keys of its own block of ``chunk`` cache slots,
     ``floor(j / chunk) == floor(i / chunk)`` (blocks count from slot 0 of the row, wherever a prompt was cut).
-    ``head_scale [H]``: the score of head ``h`` is also multiplied by ``head_scale[h]`` (before cap and bias). ``kc`` and
-    ``vc`` may be one tensor (latent attention). Returns fp32 ``[B*S, H*vdim]``."""
+    ``head_scale [H]``: the score of head ``h`` is also multiplied by ``head_scale[h]`` (before cap and bias).
+    ``window > 0``: query ``i`` sees key ``j <= i`` only if ``i - j < window`` or ``j < keep_first`` (the first
+    ``keep_first`` slots of a row stay visible to every later query). ``gate [B*S, >= H]`` (a column view is fine): head
+    ``h``'s output of token ``m`` is multiplied by ``sigmoid(gate[m, h])``. ``kc`` and ``vc`` may be one tensor (latent
+    attention); ``vdim``: the values are the first ``vdim`` columns of ``vc``'s rows. Returns fp32 ``[B*S, H*vdim]``."""
     b, s, h, dim = q.shape
-    g, vdim = kc.shape[1], vc.shape[3]
+    g = kc.shape[1]
+    vdim = vc.shape[3] if vdim is None else int(vdim)
+    if chunk and window:
+        raise ValueError("attn_bias: a block-local mask and a sliding window exclude each other")
     if not _gpu(q):
         s0 = _slot_int(slot)
         t = s0 + s
         k = kc[:, :, :t].float().repeat_interleave(h // g, 1)  # [B, H, t, dim]
-        v = vc[:, :, :t].float().repeat_interleave(h // g, 1)
+        v = vc[:, :, :t, :vdim].float().repeat_interleave(h // g, 1)
         sc = torch.einsum("bshd,bhtd->bhst", q.float(), k) * scale
         if head_scale is not None:
             sc = sc * head_scale.float().reshape(1, h, 1, 1)
@@ -593,6 +760,8 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
         hidden = dist < 0
         if chunk and chunk > 0:
             hidden = hidden | (torch.div(qi, chunk, rounding_mode="floor") != torch.div(kj, chunk, rounding_mode="floor"))
+        if window and window > 0:
+            hidden = hidden | ((dist >= window) & (kj >= keep_first))
         sc = sc.masked_fill(hidden[None, None], float("-inf"))
         if sink is not None:
             sc = torch.cat([sc, sink.float().reshape(1, h, 1, 1).expand(b, h, s, 1)], -1)
@@ -600,20 +769,24 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
         else:
             pr = torch.softmax(sc, -1)
         o = torch.einsum("bhst,bhtv->bshv", pr, v)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[:, :h].float()).reshape(b, s, h, 1)
         return o.reshape(b * s, h * vdim)
     out = torch.empty(b * s, h * vdim, dtype=F32, device=q.device)
     e = ext()
     t_cap = int(max_kv) if max_kv is not None else kc.shape[2]
     ws, splits, vt = None, 1, None
     if s == 1:
-        splits = int(e.attn_decode_splits(b, h, min(t_cap, chunk) if chunk and chunk > 0 else t_cap))
+        seen = min(t_cap, chunk) if chunk and chunk > 0 else (min(t_cap, window + keep_first) if window > 0 else t_cap)
+        splits = int(e.attn_decode_splits(b, h, seen))
         ws = torch.empty(b * h * splits * (vdim + 2), dtype=F32, device=q.device)
     elif MMA_PREFILL:
-        nb = int(e.attn_prefill_ws_bytes(b, s, g, dim, vdim, kc.shape[2], kc.dtype == BF16))
+        nb = int(e.attn_prefill_ws_bytes(b, s, g, dim, vdim, kc.shape[2], kc.dtype == BF16)) if vdim == vc.shape[3] else 0
         if nb:  # bf16 caches at the MFMA shapes: the flash kernel over a transposed copy of the values
             vt = torch.empty(nb // 2, dtype=BF16, device=q.device)
     e.attn_bias(q.contiguous(), kc, vc, _slot_tensor(slot, q.device), float(scale), float(softcap or 0.0), bias, out,
-                t_cap, ws, splits, vt, sink, int(chunk or 0), head_scale)
+                t_cap, ws, splits, vt, sink, int(chunk or 0), head_scale, int(window or 0), int(keep_first or 0), gate,
+                vdim)
     return out
 
 
@@ -733,6 +906,19 @@ def _turn_cpu(x: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, sign: floa
     return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * half:]], -1)
 
 
+def _turn_pairs_cpu(x: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, sign: float = 1.0) -> torch.Tensor:
+    """Rotate the first ``2 len(freq)`` numbers of the last axis of ``x [M, heads, n]`` by ``sign * pos[m]``: number
+    ``2i`` pairs with number ``2i + 1``."""
+    half = freq.numel()
+    if half == 0:
+        return x
+    ang = pos.reshape(-1).double()[:, None] * freq.double()[None, :] * sign
+    c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+    u, v = x[..., 0:2 * half:2], x[..., 1:2 * half:2]
+    turned = torch.stack([u * c - v * s, v * c + u * s], -1).flatten(-2)
+    return torch.cat([turned, x[..., 2 * half:]], -1)
+
+
 def rope_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor, slot, b: int, s: int, heads: int,
               kv_heads: int, dim: int, vdim: int, kc: torch.Tensor, vc: torch.Tensor, qk_freq: torch.Tensor,
               v_freq: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -763,10 +949,12 @@ def rope_prep(proj: torch.Tensor, bias: Optional[torch.Tensor], positions: torch
 
 
 def rotate_heads(a: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], heads: int, sign: float = 1.0,
-                 gain: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``out [M, heads * n] = turn(a [M, heads * n], sign * position) * gain``: every head's first ``2 len(freq)``
-    numbers rotated (pairs ``i``, ``i + len(freq)``) by ``sign`` times the row's position; ``freq`` None: a scaled copy.
-    ``out`` may be a column slice of a wider buffer."""
+                 gain: float = 1.0, out: Optional[torch.Tensor] = None, offset: int = 0,
+                 interleaved: bool = False) -> torch.Tensor:
+    """``out [M, heads * n] = turn(a [M, heads * n], sign * position) * gain``: in every head the ``2 len(freq)`` numbers
+    from ``offset`` on are rotated by ``sign`` times the row's position (pairs ``i``, ``i + len(freq)``, or with
+    ``interleaved`` pairs ``2i``, ``2i + 1``); ``freq`` None: a scaled copy. ``out`` may be a column slice of a wider
+    buffer, or ``a`` itself."""
     m = a.shape[0]
     n = a.shape[1] // heads
     if out is None:
@@ -774,10 +962,12 @@ def rotate_heads(a: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.
     if not _gpu(a):
         x = a.float().reshape(m, heads, n)
         if freq is not None:
-            x = _turn_cpu(x, positions.reshape(-1), freq, sign)
+            turn = _turn_pairs_cpu if interleaved else _turn_cpu
+            x = torch.cat([x[..., :offset], turn(x[..., offset:], positions.reshape(-1), freq, sign)], -1)
         out.copy_(x.reshape(m, heads * n) * gain)
         return out
-    ext().rotate_heads(a, positions.reshape(-1).to(torch.int32).contiguous(), freq, heads, float(sign), float(gain), out)
+    ext().rotate_heads(a, positions.reshape(-1).to(torch.int32).contiguous(), freq, heads, float(sign), float(gain), out,
+                       int(offset), bool(interleaved))
     return out
 
 
