@@ -14,6 +14,12 @@
 // Block-local masks (chunk > 0): a query at slot i sees the keys of [floor(i / chunk) * chunk, i]; every kernel starts
 // its key walk at that block's first slot, so the keys before it are never read. A per-head factor (head_scale) joins
 // the score scale.
+// Sliding windows (window > 0): a query at slot i sees the keys of [max(0, i - window + 1), i] and, with keep_first, the
+// row's first keep_first slots. Every kernel numbers a query's visible keys 0 .. n - 1 (the kept first ones, then the
+// window) and walks that numbering, so hidden keys are never read and the decode splits deal only visible keys; the MFMA
+// kernel walks the kept tiles and then the window's tiles. A gate per (token, head) (sigmoid of a projection column)
+// multiplies the normalised output in the kernels that write it. Values may be the leading columns of wider rows (ldv):
+// a latent cache whose rows carry a rotated key part behind the latent serves as keys (whole row) and values (latent).
 #include "hy_util.h"
 #include "hybrid.h"
 
@@ -42,27 +48,31 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(AttnPrep p) {
   if (item < p.H) { kind = 0; head = item; len = p.dim; col = head * p.dim; }
   else if (item < p.H + p.G) { kind = 1; head = item - p.H; len = p.dim; col = p.H * p.dim + head * p.dim; }
   else { kind = 2; head = item - p.H - p.G; len = p.vdim; col = (p.H + p.G) * p.dim + head * p.vdim; }
-  float ss = 0.f;
-  for (int d = lane; d < len; d += 64) {
-    const float v = row[col + d];
-    ss = fmaf(v, v, ss);
+  float sc = 1.f;
+  if (kind != 2 || p.norm_v) {
+    float ss = 0.f;
+    for (int d = lane; d < len; d += 64) {
+      const float v = row[col + d];
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    sc = 1.f / sqrtf(ss / (float)len + p.eps);
   }
-  ss = wave_sum(ss);
-  float sc = 1.f / sqrtf(ss / (float)len + p.eps);
+  const float* gw = kind == 0 ? p.q_w : (kind == 1 ? p.k_w : nullptr);  // gain of the norm, shared by the heads
   if (kind == 0) {
     if (p.temp_coef != 0.f) {
       const int pos = p.positions[m];
       sc *= 1.f + p.temp_coef * logf((float)((pos + 1) / p.temp_every) + 1.f);
     }
     float* q = p.q + ((size_t)m * p.H + head) * p.dim;
-    for (int d = lane; d < len; d += 64) q[d] = row[col + d] * sc;
+    for (int d = lane; d < len; d += 64) q[d] = row[col + d] * sc * (gw ? gw[d] : 1.f);
     return;
   }
   const int t = *p.slot + sidx;
   if (t < 0 || t >= p.T) return;  // cache full: the write is dropped
   CT* dst = (kind == 1 ? reinterpret_cast<CT*>(p.kc) : reinterpret_cast<CT*>(p.vc)) +
             (((size_t)b * p.G + head) * p.T + t) * len;
-  for (int d = lane; d < len; d += 64) ab_st(dst + d, row[col + d] * sc);
+  for (int d = lane; d < len; d += 64) ab_st(dst + d, row[col + d] * sc * (gw ? gw[d] : 1.f));
 }
 
 int hy_attn_prep(const AttnPrep& p, hipStream_t s) {
@@ -82,16 +92,31 @@ int hy_attn_prep(const AttnPrep& p, hipStream_t s) {
 constexpr int AB_MAX_DIM = 512;   // q head held in LDS per wave
 constexpr int AB_MAX_VREG = 8;    // value columns per lane: vdim <= 512
 
-// One wave: keys [j_lo, j_hi) of query (b, h) at slot qi; returns the running max m, sum l and unnormalised acc.
-// with_sink: the wave whose keys start the row also counts the head's sink.
+// The keys a query at slot qi sees: slots [0, kf) (kept first keys, only beside a window) and [lo, qi], numbered
+// 0 .. n - 1 in that order.
+struct AbSpan {
+  int kf, lo, n;
+};
+JLA_DEV AbSpan ab_span(const AttnBias& p, int qi) {
+  AbSpan sp;
+  sp.lo = p.chunk > 0 ? qi / p.chunk * p.chunk : (p.window > 0 ? max(0, qi - p.window + 1) : 0);
+  sp.kf = p.window > 0 ? min(p.keep_first, sp.lo) : 0;
+  sp.n = sp.kf + qi + 1 - sp.lo;
+  return sp;
+}
+JLA_DEV int ab_key(const AbSpan& sp, int v) { return v < sp.kf ? v : sp.lo + (v - sp.kf); }
+JLA_DEV float ab_gate(const AttnBias& p, size_t m, int h) { return p.gate ? hy_sigmoid(p.gate[m * p.ldg + h]) : 1.f; }
+
+// One wave: visible keys number [j_lo, j_hi) of query (b, h) at slot qi (span); returns the running max m, sum l and
+// unnormalised acc. with_sink: the wave whose keys start the row also counts the head's sink.
 template <typename CT, int VREG>  // VREG: value columns per lane (vdim <= 64 VREG)
-JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, int j_lo, int j_hi, bool with_sink,
-                     float& m_run, float& l_run, float* acc) {
+JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, const AbSpan& span, int j_lo, int j_hi,
+                     bool with_sink, float& m_run, float& l_run, float* acc) {
   constexpr int KB = VREG <= 2 ? 16 : 8;  // keys whose value rows are in flight at a time
   const int lane = threadIdx.x & 63;
   const int g = h / (p.H / p.G);
   const CT* kbase = reinterpret_cast<const CT*>(p.kc) + ((size_t)b * p.G + g) * p.T * p.dim;
-  const CT* vbase = reinterpret_cast<const CT*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.vdim;
+  const CT* vbase = reinterpret_cast<const CT*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.ldv;
   const bool fastk = (p.dim & 7) == 0 && ((uintptr_t)kbase & 15) == 0;
   const bool sunk = with_sink && p.sink;
   const float hs = p.head_scale ? p.head_scale[h] : 1.f;
@@ -101,9 +126,10 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
   for (int i = 0; i < VREG; ++i) acc[i] = 0.f;
   for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
     const int j = j0 + lane;
+    const int kj = ab_key(span, min(j, j_hi - 1));  // cache slot of this lane's key
     float sc = -INFINITY;
     if (j < j_hi) {
-      const CT* kr = kbase + (size_t)j * p.dim;
+      const CT* kr = kbase + (size_t)kj * p.dim;
       float d0 = 0.f, d1 = 0.f;
       if (fastk) {  // whole 16-byte groups: branch-free loads the scheduler can batch
 #pragma unroll 4
@@ -121,7 +147,7 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
       }
       sc = (d0 + d1) * p.scale * hs;
       if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
-      if (p.bias) sc += p.bias[(size_t)min(qi - j, p.nbias - 1) * p.H + h];
+      if (p.bias) sc += p.bias[(size_t)min(qi - kj, p.nbias - 1) * p.H + h];
     }
     const float m_new = fmaxf(m_run, wave_max(sc));
     const float corr = expf(m_run - m_new);  // first chunk: exp(-inf) = 0
@@ -135,7 +161,7 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
       float vv[KB][VREG];
 #pragma unroll
       for (int u = 0; u < KB; ++u) {
-        const CT* vr = vbase + (size_t)min(j0 + jj + u, j_hi - 1) * p.vdim;
+        const CT* vr = vbase + (size_t)ab_key(span, min(j0 + jj + u, j_hi - 1)) * p.ldv;
 #pragma unroll
         for (int i = 0; i < VREG; ++i) {
           vv[u][i] = ab_ld(vr + min(lane + 64 * i, p.vdim - 1));  // (columns past vdim: never stored)
@@ -152,15 +178,12 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
   }
 }
 
-// first key slot a query at slot qi sees
-JLA_DEV int ab_first_key(const AttnBias& p, int qi) { return p.chunk > 0 ? qi / p.chunk * p.chunk : 0; }
-
-// keys [j_lo, j_hi) of decode split sp: the query's visible keys [lo, qi] dealt to the splits in runs of 64
-JLA_DEV void ab_split_range(const AttnBias& p, int qi, int sp, int& j_lo, int& j_hi) {
-  const int lo = ab_first_key(p, qi), n = qi + 1 - lo;
+// visible keys number [j_lo, j_hi) of decode split sp: the query's n visible keys dealt to the splits in runs of 64
+JLA_DEV void ab_split_range(const AttnBias& p, const AbSpan& span, int sp, int& j_lo, int& j_hi) {
+  const int n = span.n;
   const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
-  j_lo = lo + min(n, sp * per);
-  j_hi = min(lo + n, j_lo + per);
+  j_lo = min(n, sp * per);
+  j_hi = min(n, j_lo + per);
 }
 
 // prefill: grid (ceil(S / 4), H, B), one wave per query
@@ -176,9 +199,10 @@ __global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
   __builtin_amdgcn_wave_barrier();
   const int qi = min(*p.slot + s, p.T - 1);
   float m_run, l_run, acc[VREG];
-  ab_wave<CT, VREG>(p, qs, b, h, qi, ab_first_key(p, qi), qi + 1, true, m_run, l_run, acc);
+  const AbSpan span = ab_span(p, qi);
+  ab_wave<CT, VREG>(p, qs, b, h, qi, span, 0, span.n, true, m_run, l_run, acc);
   float* o = p.out + ((size_t)b * p.S + s) * (p.H * p.vdim) + (size_t)h * p.vdim;
-  const float inv = 1.f / l_run;
+  const float inv = ab_gate(p, (size_t)b * p.S + s, h) / l_run;
 #pragma unroll
   for (int i = 0; i < VREG; ++i) {
     const int c = lane + 64 * i;
@@ -197,9 +221,10 @@ __global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
   __syncthreads();
   const int qi = min(*p.slot, p.T - 1);
   int j_lo, j_hi;
-  ab_split_range(p, qi, sp, j_lo, j_hi);
+  const AbSpan span = ab_span(p, qi);
+  ab_split_range(p, span, sp, j_lo, j_hi);
   float m_run, l_run, acc[VREG];
-  ab_wave<CT, VREG>(p, qs, b, h, qi, j_lo, j_hi, sp == 0, m_run, l_run, acc);
+  ab_wave<CT, VREG>(p, qs, b, h, qi, span, j_lo, j_hi, sp == 0, m_run, l_run, acc);
   float* w = p.ws + (((size_t)b * p.H + h) * p.splits + sp) * (p.vdim + 2);
   if (lane == 0) {
     w[0] = m_run;
@@ -228,9 +253,10 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
   for (int i = 0; i < dim / 64; ++i) qv[i] = q[lane + 64 * i];
   const int qi = min(*p.slot, p.T - 1);
   int j_lo, j_hi;
-  ab_split_range(p, qi, sp, j_lo, j_hi);
+  const AbSpan span = ab_span(p, qi);
+  ab_split_range(p, span, sp, j_lo, j_hi);
   const bf16_t* kbase = reinterpret_cast<const bf16_t*>(p.kc) + ((size_t)b * p.G + g) * p.T * dim;
-  const bf16_t* vbase = reinterpret_cast<const bf16_t*>(p.vc) + ((size_t)b * p.G + g) * p.T * vdim;
+  const bf16_t* vbase = reinterpret_cast<const bf16_t*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.ldv;
   const bool sunk = p.sink && sp == 0;
   const float hs = p.head_scale ? p.head_scale[h] : 1.f;
   float m_run = sunk ? p.sink[h] : -INFINITY, l_run = sunk ? 1.f : 0.f, acc[VREG];
@@ -238,7 +264,7 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
   for (int i = 0; i < VREG; ++i) acc[i] = 0.f;
   bool staged = false;
   for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
-    const int j = j0 + lane, jc = min(j, j_hi - 1);
+    const int j = j0 + lane, jc = ab_key(span, min(j, j_hi - 1));  // (jc: the cache slot)
     u32x4 kf[DK8];
 #pragma unroll
     for (int u = 0; u < DK8; ++u) kf[u] = *reinterpret_cast<const u32x4*>(kbase + (size_t)jc * dim + 8 * u);
@@ -246,7 +272,7 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
     bf16_t vv[64][VREG];
 #pragma unroll
     for (int jj = 0; jj < 64; ++jj) {
-      const bf16_t* vr = vbase + (size_t)min(j0 + jj, j_hi - 1) * vdim + lane;
+      const bf16_t* vr = vbase + (size_t)ab_key(span, min(j0 + jj, j_hi - 1)) * p.ldv + lane;
 #pragma unroll
       for (int i = 0; i < VREG; ++i) vv[jj][i] = vr[64 * i];
     }
@@ -294,8 +320,8 @@ __global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
   for (int i = 0; i < VREG; ++i) w[2 + lane + 64 * i] = acc[i];
 }
 
-// decode over a shared latent: keys = values = ONE bf16 cache head (kc == vc, G == 1), rows of 136 to 512 numbers, no
-// bias / soft cap. The lanes split a row's numbers, 16 bytes each, so one coalesced load per key serves both the score
+// decode over a shared latent: keys = values = ONE bf16 cache head (kc == vc, G == 1), rows of 136 to 512 numbers of
+// which the first vdim are the values (all of them, or a latent in front of a rotated key part), no bias / soft cap. The lanes split a row's numbers, 16 bytes each, so one coalesced load per key serves both the score
 // (row totals by DPP, the four rows through scalar registers: no LDS round trips) and the value sum; all loads of a
 // chunk of keys are issued before the first use. A wave serves HQ heads of one row (HQ = 4 measured slower than 1 at 8
 // rows x 16 heads, 94 against 58 us: four times the scalar-register traffic per key on a quarter of the waves; dealing
@@ -323,7 +349,8 @@ __global__ void __launch_bounds__(64) attn_latent_decode_kernel(AttnBias p) {
   }
   const int qi = min(*p.slot, p.T - 1);
   int j_lo, j_hi;
-  ab_split_range(p, qi, sp, j_lo, j_hi);
+  const AbSpan span = ab_span(p, qi);
+  ab_split_range(p, span, sp, j_lo, j_hi);
   const bf16_t* base = reinterpret_cast<const bf16_t*>(p.kc) + (size_t)b * p.T * rank + c0;
   const bool sunk = p.sink && sp == 0;
   float m_run[HQ], l_run[HQ], acc[HQ][8], hs[HQ];
@@ -339,7 +366,7 @@ __global__ void __launch_bounds__(64) attn_latent_decode_kernel(AttnBias p) {
     u32x4 rows[KC];
 #pragma unroll
     for (int u = 0; u < KC; ++u)
-      rows[u] = *reinterpret_cast<const u32x4*>(base + (size_t)min(j0 + u, j_hi - 1) * rank);
+      rows[u] = *reinterpret_cast<const u32x4*>(base + (size_t)ab_key(span, min(j0 + u, j_hi - 1)) * rank);
     float sc[HQ][KC], cmax[HQ];
 #pragma unroll
     for (int q = 0; q < HQ; ++q) cmax[q] = -INFINITY;
@@ -391,7 +418,7 @@ __global__ void __launch_bounds__(64) attn_latent_decode_kernel(AttnBias p) {
       w[0] = m_run[q];
       w[1] = l_run[q];
     }
-    if (on) {
+    if (on && c0 < p.vdim) {  // (the values are the row's first vdim numbers)
 #pragma unroll
       for (int i = 0; i < 8; ++i) w[2 + c0 + i] = acc[q][i];
     }
@@ -422,7 +449,7 @@ __global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
     const float ws = __shfl(wt, sp, 64);
     a = fmaf(part[sp], sp < p.splits ? ws : 0.f, a);
   }
-  if (c0 + lane < p.vdim) o[c] = a / l;
+  if (c0 + lane < p.vdim) o[c] = a / l * ab_gate(p, b, h);
 }
 
 // ---- MFMA flash prefill (bf16 caches) ----------------------------------------------------------------------------------
@@ -499,8 +526,12 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
   const float inv_cap = p.softcap > 0.f ? 1.f / p.softcap : 0.f;
   const float hs = p.head_scale ? p.head_scale[h] : 1.f;
   // block-local mask: this query's first key, the last query's (the largest of the wave), and the tile the walk starts at
-  const int lo_q = ab_first_key(p, qi), lo_last = ab_first_key(p, q_last);
-  const int j_begin = ab_first_key(p, q0) / AM_K * AM_K;
+  const int lo_q = ab_span(p, qi).lo, lo_last = ab_span(p, q_last).lo;
+  const int j_begin = ab_span(p, q0).lo / AM_K * AM_K;
+  // kept first keys (beside a window): their tiles [0, kf_end) come first, then the walk jumps to the window's tiles
+  const int kfirst = p.window > 0 ? p.keep_first : 0;
+  const int kf_end = min((kfirst + AM_K - 1) / AM_K * AM_K, j_begin);
+  auto next_tile = [&](int j0) { return j0 + AM_K == kf_end ? j_begin : j0 + AM_K; };
   // the next tile's key and value fragments are loaded while the current tile is computed (one wave per SIMD at small
   // batch: nothing else hides the loads)
   u32x4 kn[DK], vn[2][VT];
@@ -514,8 +545,9 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
       for (int v = 0; v < VT; ++v)
         vn[c][v] = *reinterpret_cast<const u32x4*>(vbase + (size_t)(32 * v + ql) * Tp + min(j0, Tp - AM_K) + 16 * c + 8 * hi);
   };
-  fetch(j_begin);
-  for (int j0 = j_begin; j0 <= q_last; j0 += AM_K) {
+  const int j_first = kf_end > 0 ? 0 : j_begin;
+  fetch(j_first);
+  for (int j0 = j_first; j0 <= q_last; j0 = next_tile(j0)) {
     u32x4 kc_[DK], vc_[2][VT];
 #pragma unroll
     for (int kk = 0; kk < DK; ++kk) kc_[kk] = kn[kk];
@@ -523,7 +555,7 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int v = 0; v < VT; ++v) vc_[c][v] = vn[c][v];
-    fetch(j0 + AM_K);  // (past the last tile: clamped addresses, never used)
+    fetch(next_tile(j0));  // (past the last tile: clamped addresses, never used)
     // scores: rows = keys (fed permuted), columns = queries
     f32x16 sacc;
 #pragma unroll
@@ -536,7 +568,8 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
     const int dbase = q0 - j0 - (AM_K - 1);
     const bool far = p.bias && dbase >= p.nbias - 1;
     if (p.bias) bl = p.bias[(size_t)min(max(dbase + lane, 0), p.nbias - 1) * p.H + h];
-    const bool diag = j0 + AM_K - 1 > q0 || j0 < lo_last;  // some (query, key) of the tile is masked
+    // some (query, key) of the tile is masked
+    const bool diag = j0 + AM_K - 1 > q0 || (j0 < lo_last && j0 + AM_K - 1 >= kfirst);
     float tmax = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -544,7 +577,7 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
       float sc = sacc[r] * p.scale * hs;
       if (p.softcap > 0.f) sc = p.softcap * am_tanh(sc * inv_cap);
       if (p.bias) sc += far ? bl : __shfl(bl, ql - kl + (AM_K - 1), 64);
-      if (diag && (j0 + kl > qi || j0 + kl < lo_q)) sc = -INFINITY;
+      if (diag && (j0 + kl > qi || (j0 + kl < lo_q && j0 + kl >= kfirst))) sc = -INFINITY;
       sacc[r] = sc;
       tmax = fmaxf(tmax, sc);
     }
@@ -585,7 +618,7 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
   }
   l_run += __shfl_xor(l_run, 32, 64);
   if (s0 + ql >= p.S) return;
-  const float inv = 1.f / l_run;
+  const float inv = ab_gate(p, (size_t)b * p.S + s0 + ql, h) / l_run;
   float* out = p.out + ((size_t)b * p.S + s0 + ql) * (p.H * vdim) + (size_t)h * vdim;
 #pragma unroll
   for (int v = 0; v < VT; ++v)
@@ -646,20 +679,22 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
   if (p.B < 0 || p.S < 1 || p.H < 1 || p.G < 1 || p.H % p.G || p.T < 1) return -1;
   if (p.dim < 1 || p.dim > AB_MAX_DIM || p.vdim < 1 || p.vdim > 64 * AB_MAX_VREG) return -2;
   if (p.bias && p.nbias < 1) return -3;
-  if (p.chunk < 0) return -7;
+  if (p.chunk < 0 || p.window < 0 || p.keep_first < 0 || (p.chunk > 0 && p.window > 0)) return -7;
+  if (p.ldv < p.vdim || (p.gate && p.ldg < p.H)) return -8;
   if (p.B == 0) return 0;
   if (p.H > 65535 || p.B > 65535) return -4;
   if (p.S == 1) {
     if (p.splits < 1 || !p.ws) return -5;
     if (p.splits > 64) return -6;  // (the merge holds one split per lane)
     dim3 grid(p.splits, p.H, p.B);
-    if (p.cbf16 && (p.dim == 64 || p.dim == 128) && (p.vdim == 64 || p.vdim == 128)) {
+    if (p.cbf16 && (p.dim == 64 || p.dim == 128) && (p.vdim == 64 || p.vdim == 128) && p.ldv == p.vdim) {
       if (p.dim == 64 && p.vdim == 64) attn_bias_decode_fast_kernel<8, 1><<<grid, 64, 0, s>>>(p);
       else if (p.dim == 64) attn_bias_decode_fast_kernel<8, 2><<<grid, 64, 0, s>>>(p);
       else if (p.vdim == 64) attn_bias_decode_fast_kernel<16, 1><<<grid, 64, 0, s>>>(p);
       else attn_bias_decode_fast_kernel<16, 2><<<grid, 64, 0, s>>>(p);
-    } else if (p.cbf16 && p.kc == p.vc && p.G == 1 && p.dim == p.vdim && p.dim % 8 == 0 && p.dim > 128 &&
-               p.dim <= 512 && !p.bias && p.softcap <= 0.f && ((uintptr_t)p.kc & 15) == 0) {
+    } else if (p.cbf16 && p.kc == p.vc && p.G == 1 && p.ldv == p.dim && p.vdim <= p.dim && p.vdim % 8 == 0 &&
+               p.dim % 8 == 0 && p.dim > 128 && p.dim <= 512 && !p.bias && p.softcap <= 0.f &&
+               ((uintptr_t)p.kc & 15) == 0) {
       attn_latent_decode_kernel<1, AL_KC><<<grid, 64, 0, s>>>(p);
     } else {
       AB_BY_VREG(attn_bias_decode_kernel, grid, 64);
@@ -669,7 +704,7 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
     JLA_CHECK_LAUNCH();
     return 0;
   }
-  if (p.vt_ws && hy_attn_prefill_ws_bytes(p.B, p.S, p.G, p.dim, p.vdim, p.T, p.cbf16) > 0) {
+  if (p.vt_ws && p.ldv == p.vdim && hy_attn_prefill_ws_bytes(p.B, p.S, p.G, p.dim, p.vdim, p.T, p.cbf16) > 0) {
     const int Tp = (p.T + 31) / 32 * 32;
     bf16_t* vt = reinterpret_cast<bf16_t*>(p.vt_ws);
     if (p.dim == 64 && p.vdim == 64) return am_launch<4, 2>(p, vt, Tp, s);

@@ -65,12 +65,13 @@ const float* rows2d(const Tensor& t, const char* name, int64_t cols, int* ld) {
   return reinterpret_cast<const float*>(t.data_ptr());
 }
 
-void embed_rows(Tensor ids, Tensor table, int64_t col0, Tensor out, double scale) {
+void embed_rows(Tensor ids, Tensor table, int64_t col0, Tensor out, double scale, int64_t copies) {
   const int wb = wtype(table, "table");
-  check(table.dim() == 2 && out.dim() == 2, "embed_rows: 2-d table and out");
-  const int M = out.size(0), D = out.size(1);
+  check(table.dim() == 2 && out.dim() == 2 && copies >= 1 && out.size(0) % copies == 0,
+        "embed_rows: 2-d table, out is [copies * M, D]");
+  const int M = out.size(0) / copies, D = out.size(1);
   rc(jla::hy_embed_rows(i32(ids, "ids", M), table.data_ptr(), wb, table.size(0), table.size(1), col0,
-                        (float)scale, f32w(out, "out"), M, D, stream()),
+                        (float)scale, f32w(out, "out"), M, D, copies, stream()),
      "embed_rows");
 }
 
@@ -155,6 +156,67 @@ void route_topk(Tensor z, int64_t E, int64_t top, Tensor row_expert, Tensor row_
      "route_topk");
 }
 
+void route_grouped(Tensor z, OptT correction, int64_t E, int64_t top, int64_t groups, int64_t keep, Tensor row_expert,
+                   Tensor row_tok, Tensor row_w, OptT sort_tok, OptT sort_dst, OptT sort_w, OptT offs) {
+  check(z.dim() == 2 && z.size(1) >= E && top >= 1 && top <= E, "route_grouped: z is [M, >= E], 1 <= top <= E");
+  int ldz = 0;
+  const float* zp = rows2d(z, "z", z.size(1), &ldz);
+  const int M = z.size(0);
+  const int64_t R = (int64_t)M * top;
+  check(row_w.numel() >= R, "route_grouped: weight outputs hold R numbers");
+  check(!correction.has_value() || correction->numel() == E, "route_grouped: correction is [E]");
+  const bool sorted = sort_tok.has_value();
+  check(sorted == sort_dst.has_value() && sorted == sort_w.has_value() && sorted == offs.has_value(),
+        "route_grouped: the sorted outputs come together");
+  check(!sorted || sort_w->numel() >= R, "route_grouped: weight outputs hold R numbers");
+  rc(jla::hy_route_grouped(zp, ldz, correction.has_value() ? f32(*correction, "correction") : nullptr, M, top, E, groups,
+                           keep, i32w(row_expert, "row_expert", R), i32w(row_tok, "row_tok", R), f32w(row_w, "row_w"),
+                           sorted ? i32w(*sort_tok, "sort_tok", R) : nullptr,
+                           sorted ? i32w(*sort_dst, "sort_dst", R) : nullptr, sorted ? f32w(*sort_w, "sort_w") : nullptr,
+                           sorted ? i32w(*offs, "offs", E + 1) : nullptr, stream()),
+     "route_grouped");
+}
+
+void hc_update(Tensor xs, OptT mix, OptT out_w, OptT y, int64_t nsum, OptT row_w, OptT row_expert, int64_t n_real,
+               OptT ident, OptT extra, OptT next_in, OptT u) {
+  jla::HyperUpdate p{};
+  check(xs.dim() == 3, "hc_update: xs is [S, M, D]");
+  p.S = xs.size(0); p.M = xs.size(1); p.D = xs.size(2);
+  p.xs = f32w(xs, "xs");
+  const int64_t md = (int64_t)p.M * p.D;
+  check(mix.has_value() == out_w.has_value() && mix.has_value() == y.has_value(), "hc_update: mix, out_w and y together");
+  if (mix.has_value()) {
+    check(mix->numel() == (int64_t)p.S * p.S && out_w->numel() == p.S, "hc_update: mix is [S, S], out_w [S]");
+    p.mix = f32(*mix, "mix");
+    p.out_w = f32(*out_w, "out_w");
+    check(nsum >= 1 && y->numel() == md * nsum, "hc_update: y is [M * nsum, D]");
+    p.y = f32(*y, "y");
+    p.nsum = nsum;
+    const int64_t R = (int64_t)p.M * nsum;
+    if (row_w.has_value()) {
+      check(row_w->numel() >= R, "hc_update: row_w is [M * nsum]");
+      p.row_w = f32(*row_w, "row_w");
+    }
+    if (row_expert.has_value()) {
+      check(row_w.has_value() && ident.has_value() && ident->numel() == md, "hc_update: row_expert needs row_w and ident [M, D]");
+      p.row_expert = i32(*row_expert, "row_expert", R);
+      p.ident = f32(*ident, "ident");
+      p.n_real = n_real;
+    }
+    if (extra.has_value()) {
+      check(extra->numel() == md, "hc_update: extra is [M, D]");
+      p.extra = f32(*extra, "extra");
+    }
+  }
+  check(next_in.has_value() == u.has_value(), "hc_update: next_in and u together");
+  if (next_in.has_value()) {
+    check(next_in->numel() == p.S && u->numel() == md, "hc_update: next_in is [S], u [M, D]");
+    p.next_in = f32(*next_in, "next_in");
+    p.u = f32w(*u, "u");
+  }
+  rc(jla::hy_hc_update(p, stream()), "hc_update");
+}
+
 void norm_residual(Tensor y, int64_t nsum, double ysc, Tensor w, double eps, OptT x, OptT out, OptT extra,
                    OptT extra_gate) {
   check(y.dim() == 2 && nsum >= 1 && y.size(0) % nsum == 0, "norm_residual: y is [M * nsum, D]");
@@ -207,8 +269,18 @@ void gelu_gate_rows(Tensor gp, Tensor ids, Tensor table, int64_t col0, Tensor g)
 }
 
 void attn_prep(Tensor proj, Tensor positions, Tensor slot, int64_t B, int64_t S, int64_t H, int64_t G, int64_t dim,
-               int64_t vdim, OptT kc, OptT vc, Tensor q, double eps, double temp_coef, int64_t temp_every) {
+               int64_t vdim, OptT kc, OptT vc, Tensor q, double eps, double temp_coef, int64_t temp_every, OptT q_w, OptT k_w,
+               bool norm_v) {
   jla::AttnPrep p{};
+  p.norm_v = norm_v;
+  if (q_w.has_value()) {
+    check(q_w->numel() == dim, "attn_prep: q_w is [dim]");
+    p.q_w = f32(*q_w, "q_w");
+  }
+  if (k_w.has_value()) {
+    check(k_w->numel() == dim, "attn_prep: k_w is [dim]");
+    p.k_w = f32(*k_w, "k_w");
+  }
   p.has_kv = kc.has_value();
   check(kc.has_value() == vc.has_value(), "attn_prep: k and v caches together");
   const int64_t cols = H * dim + (p.has_kv ? G * (dim + vdim) : 0);
@@ -236,8 +308,10 @@ void attn_prep(Tensor proj, Tensor positions, Tensor slot, int64_t B, int64_t S,
   rc(jla::hy_attn_prep(p, stream()), "attn_prep");
 }
 
+const double* f64(const Tensor& t, const char* name);
+
 void latent_prep(Tensor proj, int64_t col0, Tensor w, Tensor slot, int64_t B, int64_t S, Tensor cache, double eps,
-                 OptT q) {
+                 OptT q, int64_t q_col0, OptT q_norm_w, OptT rot_freq, OptT positions) {
   jla::LatentPrep p{};
   check(proj.dim() == 2 && proj.size(0) == B * S && proj.scalar_type() == torch::kFloat32 && proj.is_cuda() &&
             proj.stride(1) == 1,
@@ -246,19 +320,32 @@ void latent_prep(Tensor proj, int64_t col0, Tensor w, Tensor slot, int64_t B, in
   p.ld = proj.stride(0);
   p.col0 = col0;
   p.cbf16 = wtype(cache, "latent cache");
-  check(cache.dim() == 4 && cache.size(0) == B && cache.size(1) == 1, "latent_prep: cache is [B, 1, T, rank]");
+  check(cache.dim() == 4 && cache.size(0) == B && cache.size(1) == 1, "latent_prep: cache is [B, 1, T, row]");
   p.T = cache.size(2);
-  p.rank = cache.size(3);
-  check(col0 >= 0 && col0 + p.rank <= proj.size(1) && w.numel() == p.rank, "latent_prep: latent columns / gain");
+  p.row = cache.size(3);
+  p.rank = w.numel();
+  check(col0 >= 0 && p.rank >= 1 && p.rank <= p.row && col0 + p.row <= proj.size(1), "latent_prep: latent columns / gain");
+  if (rot_freq.has_value() && rot_freq->numel() > 0) {
+    p.rot_half = rot_freq->numel();
+    check(2 * p.rot_half <= p.row - p.rank && positions.has_value(), "latent_prep: rotated numbers / positions");
+    p.rot_freq = f64(*rot_freq, "rot_freq");
+    p.positions = i32(*positions, "positions", B * S);
+  }
   p.w = f32(w, "w");
   p.slot = i32(slot, "slot", 1);
   p.B = B; p.S = S;
   p.cache = cache.data_ptr();
   p.eps = eps;
   if (q.has_value()) {
-    check(q->dim() == 2 && q->size(0) == B * S && q->size(1) <= proj.size(1), "latent_prep: q is [B * S, q_cols]");
+    check(q->dim() == 2 && q->size(0) == B * S && q_col0 >= 0 && q_col0 + q->size(1) <= proj.size(1),
+          "latent_prep: q is [B * S, q_cols]");
     p.q = f32w(*q, "q");
     p.q_cols = q->size(1);
+    p.q_col0 = q_col0;
+    if (q_norm_w.has_value()) {
+      check(q_norm_w->numel() == p.q_cols, "latent_prep: q_norm_w is [q_cols]");
+      p.q_norm_w = f32(*q_norm_w, "q_norm_w");
+    }
   }
   rc(jla::hy_latent_prep(p, stream()), "latent_prep");
 }
@@ -270,7 +357,8 @@ int64_t attn_prefill_ws_bytes(int64_t B, int64_t S, int64_t G, int64_t dim, int6
 }
 
 void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double softcap, OptT bias, Tensor out,
-               int64_t t_cap, OptT ws, int64_t splits, OptT vt_ws, OptT sink, int64_t chunk, OptT head_scale) {
+               int64_t t_cap, OptT ws, int64_t splits, OptT vt_ws, OptT sink, int64_t chunk, OptT head_scale, int64_t window,
+               int64_t keep_first, OptT gate, c10::optional<int64_t> vdim) {
   jla::AttnBias p{};
   check(q.dim() == 4, "attn_bias: q is [B, S, H, dim]");
   p.B = q.size(0); p.S = q.size(1); p.H = q.size(2); p.dim = q.size(3);
@@ -280,7 +368,17 @@ void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double
   check(kc.dim() == 4 && vc.dim() == 4 && kc.size(0) == p.B && vc.size(0) == p.B && kc.size(3) == p.dim &&
             kc.size(1) == vc.size(1) && kc.size(2) == vc.size(2),
         "attn_bias: cache shapes");
-  p.G = kc.size(1); p.T = kc.size(2); p.vdim = vc.size(3);
+  p.G = kc.size(1); p.T = kc.size(2);
+  p.ldv = vc.size(3);
+  p.vdim = vdim.has_value() ? *vdim : vc.size(3);
+  check(p.vdim >= 1 && p.vdim <= p.ldv, "attn_bias: vdim is at most the width of a value row");
+  check(window >= 0 && window <= INT32_MAX && keep_first >= 0 && keep_first <= INT32_MAX, "attn_bias: window / keep_first");
+  p.window = window;
+  p.keep_first = keep_first;
+  if (gate.has_value()) {
+    check(gate->dim() == 2 && gate->size(0) == (int64_t)p.B * p.S && gate->size(1) >= p.H, "attn_bias: gate is [B * S, >= H]");
+    p.gate = rows2d(*gate, "gate", gate->size(1), &p.ldg);
+  }
   p.kc = kc.data_ptr();
   p.vc = vc.data_ptr();
   p.slot = i32(slot, "slot", 1);
@@ -461,16 +559,17 @@ void rope_prep(Tensor proj, OptT bias, Tensor positions, Tensor slot, int64_t B,
   rc(jla::hy_rope_prep(p, stream()), "rope_prep");
 }
 
-void rotate_heads(Tensor a, Tensor positions, OptT freq, int64_t H, double sign, double gain, Tensor out) {
+void rotate_heads(Tensor a, Tensor positions, OptT freq, int64_t H, double sign, double gain, Tensor out, int64_t offset,
+                  bool interleaved) {
   check(a.dim() == 2 && a.size(1) % H == 0, "rotate_heads: a is [M, H * n]");
   const int64_t M = a.size(0), n = a.size(1) / H;
   int lda = 0, ldo = 0;
   const float* ap = slice2d(a, "a", M, H * n, &lda);
   float* op = slice2d(out, "out", M, H * n, &ldo);
   const int half = freq.has_value() ? (int)freq->numel() : 0;
-  check(2 * half <= n, "rotate_heads: more rotated numbers than a head holds");
+  check(offset >= 0 && offset + 2 * half <= n, "rotate_heads: more rotated numbers than a head holds");
   rc(jla::hy_rotate_heads(ap, lda, i32(positions, "positions", M), half ? f64(*freq, "freq") : nullptr, half, M, H, n,
-                          (float)sign, (float)gain, op, ldo, stream()),
+                          (float)sign, (float)gain, op, ldo, offset, interleaved, stream()),
      "rotate_heads");
 }
 
@@ -541,7 +640,10 @@ void lin_scan(int64_t mode, Tensor q, Tensor k, Tensor v, Tensor decay, OptT wri
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.attr("GEMV_MAX_R") = jla::HY_GEMV_MAX_R;
-  m.def("embed_rows", &embed_rows);
+  m.def("embed_rows", &embed_rows, py::arg("ids"), py::arg("table"), py::arg("col0"), py::arg("out"), py::arg("scale"),
+        py::arg("copies") = 1);
+  m.def("route_grouped", &route_grouped);
+  m.def("hc_update", &hc_update);
   m.def("linear_rows", &linear_rows, py::arg("a"), py::arg("a_idx"), py::arg("w"), py::arg("out"), py::arg("dst_idx"),
         py::arg("offs"), py::arg("row_expert"), py::arg("R"), py::arg("act"), py::arg("act_limit"), py::arg("act_alpha"),
         py::arg("a_scale"), py::arg("a_norm_w"), py::arg("a_norm_eps"), py::arg("even_rows") = 0,
@@ -549,7 +651,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("route_table", &route_table);
   m.def("route_topk", &route_topk);
   m.def("dense_is_gemv", &dense_is_gemv);
-  m.def("latent_prep", &latent_prep);
+  m.def("latent_prep", &latent_prep, py::arg("proj"), py::arg("col0"), py::arg("w"), py::arg("slot"), py::arg("B"),
+        py::arg("S"), py::arg("cache"), py::arg("eps"), py::arg("q"), py::arg("q_col0") = 0,
+        py::arg("q_norm_w") = py::none(), py::arg("rot_freq") = py::none(), py::arg("positions") = py::none());
   m.attr("ACT_NONE") = (int)jla::HY_ACT_NONE;
   m.attr("ACT_RELU2") = (int)jla::HY_ACT_RELU2;
   m.attr("ACT_SWIGLU") = (int)jla::HY_ACT_SWIGLU;
@@ -558,11 +662,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gelu_gate_rows", &gelu_gate_rows);
   m.def("cast_bf16", &cast_bf16);
   m.def("softcap", &softcap);
-  m.def("attn_prep", &attn_prep);
+  m.def("attn_prep", &attn_prep, py::arg("proj"), py::arg("positions"), py::arg("slot"), py::arg("B"), py::arg("S"),
+        py::arg("H"), py::arg("G"), py::arg("dim"), py::arg("vdim"), py::arg("kc"), py::arg("vc"), py::arg("q"),
+        py::arg("eps"), py::arg("temp_coef"), py::arg("temp_every"), py::arg("q_w") = py::none(),
+        py::arg("k_w") = py::none(), py::arg("norm_v") = true);
   m.def("attn_decode_splits", &attn_decode_splits);
   m.def("attn_bias", &attn_bias, py::arg("q"), py::arg("kc"), py::arg("vc"), py::arg("slot"), py::arg("scale"),
         py::arg("softcap"), py::arg("bias"), py::arg("out"), py::arg("t_cap"), py::arg("ws"), py::arg("splits"),
-        py::arg("vt_ws"), py::arg("sink"), py::arg("chunk") = 0, py::arg("head_scale") = py::none());
+        py::arg("vt_ws"), py::arg("sink"), py::arg("chunk") = 0, py::arg("head_scale") = py::none(),
+        py::arg("window") = 0, py::arg("keep_first") = 0, py::arg("gate") = py::none(), py::arg("vdim") = py::none());
   m.def("attn_prefill_ws_bytes", &attn_prefill_ws_bytes);
   m.def("delta_prep", &delta_prep);
   m.def("conv_state_update", &conv_state_update);
@@ -572,7 +680,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("gain") = 1.0);
   m.attr("ACT_SOFTCAP") = (int)jla::HY_ACT_SOFTCAP;
   m.def("rope_prep", &rope_prep);
-  m.def("rotate_heads", &rotate_heads);
+  m.def("rotate_heads", &rotate_heads, py::arg("a"), py::arg("positions"), py::arg("freq"), py::arg("H"), py::arg("sign"),
+        py::arg("gain"), py::arg("out"), py::arg("offset") = 0, py::arg("interleaved") = false);
   m.def("token_shift", &token_shift);
   m.def("mlstm_prep", &mlstm_prep);
   m.def("lin_scan", &lin_scan, py::arg("mode"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("decay"),

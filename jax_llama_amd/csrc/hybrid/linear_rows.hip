@@ -239,6 +239,7 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
     g1 = p.offs[e + 1];
   } else if (p.row_expert) {
     e = p.row_expert[g0];
+    if (e < 0 || e >= p.E) return;  // (a row of an expert without weights, an identity expert: nothing to compute)
   }
   const int K = p.K;
   for (int r0 = g0; r0 < g1; r0 += MAXR) {  // (more than MAXR rows: the weights are streamed again per 8 rows)
@@ -541,6 +542,127 @@ __global__ void __launch_bounds__(256) route_topk_select_kernel(const float* z, 
       row_w[r] = hy_sigmoid(best);
     }
   }
+}
+
+__global__ void route_sort_kernel(int R, int top, int E, const int32_t* row_expert, const float* row_w, int32_t* sort_tok,
+                                  int32_t* sort_dst, float* sort_w, int32_t* offs);
+
+// Grouped softmax router, selection: one wave per token, logits in registers as above. Scores = softmax over all E
+// logits; choice = score + correction; a group's score is its largest choice; experts outside the `keep` best groups
+// are retired before the `top` rounds. The weight of a chosen expert is its score (without the correction).
+JLA_DEV void rk_argmax(float& best, int& bi) {  // wave-wide (value, then lower index)
+#pragma unroll
+  for (int off = 32; off; off >>= 1) {
+    const float ob = __shfl_xor(best, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    if (ob > best || (ob == best && oi < bi)) {
+      best = ob;
+      bi = oi;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) route_grouped_select_kernel(const float* z, int ldz, const float* correction, int M,
+                                                                   int top, int E, int groups, int keep,
+                                                                   int32_t* row_expert, int32_t* row_tok, float* row_w) {
+  const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;
+  const float* zr = z + (size_t)m * ldz;
+  float sc[RK_PER_LANE], ch[RK_PER_LANE];
+  float zmax = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < RK_PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    const float f = e < E ? zr[e] : -INFINITY;
+    sc[u] = f == f ? f : -INFINITY;  // (a NaN logit counts as minus infinity)
+    zmax = fmaxf(zmax, sc[u]);
+  }
+  zmax = wave_max(zmax);
+  float den = 0.f;
+#pragma unroll
+  for (int u = 0; u < RK_PER_LANE; ++u) {
+    sc[u] = lane + 64 * u < E ? expf(sc[u] - zmax) : 0.f;
+    den += sc[u];
+  }
+  den = wave_sum(den);
+#pragma unroll
+  for (int u = 0; u < RK_PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    sc[u] = sc[u] / den;
+    ch[u] = e < E ? sc[u] + (correction ? correction[e] : 0.f) : -INFINITY;
+  }
+  if (groups > 1) {
+    // lane g < groups holds group g's score; `keep` rounds mark the best groups
+    const int per = E / groups;
+    float gs = -INFINITY;
+    for (int g = 0; g < groups; ++g) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < RK_PER_LANE; ++u) {
+        const int e = lane + 64 * u;
+        if (e < E && e / per == g) mx = fmaxf(mx, ch[u]);
+      }
+      mx = wave_max(mx);
+      if (lane == g) gs = mx;
+    }
+    unsigned long long kept = 0ull;
+    for (int c = 0; c < keep; ++c) {
+      float best = lane < groups && !((kept >> lane) & 1ull) ? gs : -INFINITY;
+      int bi = lane < groups && !((kept >> lane) & 1ull) ? lane : 0x7fffffff;
+      rk_argmax(best, bi);
+      if (bi != 0x7fffffff) kept |= 1ull << bi;
+    }
+#pragma unroll
+    for (int u = 0; u < RK_PER_LANE; ++u) {
+      const int e = lane + 64 * u;
+      if (e < E && !((kept >> (e / per)) & 1ull)) ch[u] = -INFINITY;
+    }
+  }
+  unsigned taken[RK_PER_LANE / 32 + 1] = {0};
+  for (int c = 0; c < top; ++c) {
+    float best = -INFINITY, bw = 0.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int u = 0; u < RK_PER_LANE; ++u) {
+      const int e = lane + 64 * u;
+      const bool free_ = !((taken[u >> 5] >> (u & 31)) & 1u);
+      if (e < E && free_ && ch[u] != -INFINITY && (ch[u] > best || (ch[u] == best && e < bi))) {
+        best = ch[u];
+        bi = e;
+      }
+    }
+    rk_argmax(best, bi);
+    if (bi == 0x7fffffff) bi = 0;  // fewer than `top` eligible experts (the host checks the sizes): expert 0, weight 0
+#pragma unroll
+    for (int u = 0; u < RK_PER_LANE; ++u)
+      if (lane + 64 * u == bi) {
+        taken[u >> 5] |= 1u << (u & 31);
+        bw = best == -INFINITY ? 0.f : sc[u];
+      }
+    bw = wave_sum(bw);  // (one lane holds the chosen expert's score)
+    if (lane == 0) {
+      const int r = m * top + c;
+      row_expert[r] = bi;
+      row_tok[r] = m;
+      row_w[r] = bw;
+    }
+  }
+}
+
+int hy_route_grouped(const float* z, int ldz, const float* correction, int M, int top, int E, int groups, int keep,
+                     int32_t* row_expert, int32_t* row_tok, float* row_w, int32_t* sort_tok, int32_t* sort_dst,
+                     float* sort_w, int32_t* offs, hipStream_t s) {
+  if (M < 0 || top < 1 || E < 1 || E > RT_MAX_E || ldz < E) return -1;
+  if (groups < 1 || groups > 64 || E % groups || keep < 1 || keep > groups || top > keep * (E / groups)) return -3;
+  if (M == 0) return 0;
+  route_grouped_select_kernel<<<(M + 3) / 4, 256, 0, s>>>(z, ldz, correction, M, top, E, groups, keep, row_expert, row_tok,
+                                                          row_w);
+  JLA_CHECK_LAUNCH();
+  if (!sort_tok) return 0;
+  if (!sort_dst || !sort_w || !offs) return -2;
+  route_sort_kernel<<<1, 256, 0, s>>>(M * top, top, E, row_expert, row_w, sort_tok, sort_dst, sort_w, offs);
+  JLA_CHECK_LAUNCH();
+  return 0;
 }
 
 __global__ void __launch_bounds__(256) route_sort_kernel(int R, int top, int E, const int32_t* row_expert,

@@ -7,7 +7,9 @@
 //                     2 qk_half numbers, optionally v heads rotated over 2 v_half numbers, q to a dense buffer, k / v into
 //                     the caches at slot + s.
 //   hy_rotate_heads : every head of a [M, H * n] activation rotated by sign * position and scaled (the inverse turn of
-//                     an attention output whose values were cached rotated), written to a column slice.
+//                     an attention output whose values were cached rotated), written to a column slice. The rotated
+//                     numbers may start at an offset within the head and may pair up as (2i, 2i + 1) instead (the
+//                     interleaved layout: the rotated tail of a latent attention's queries, in place).
 #include "hy_util.h"
 #include "hybrid.h"
 
@@ -80,33 +82,40 @@ int hy_rope_prep(const RopePrep& p, hipStream_t s) {
 }
 
 // grid (M, ceil(H / 4)), one wave per (token, head)
-__global__ void __launch_bounds__(256) rotate_heads_kernel(const float* __restrict__ a, int lda,
+__global__ void __launch_bounds__(256) rotate_heads_kernel(const float* a, int lda,
                                                            const int32_t* __restrict__ positions,
                                                            const double* __restrict__ freq, int half, int H, int n,
-                                                           float sign, float gain, float* __restrict__ out, int ldo) {
+                                                           float sign, float gain, float* out, int ldo,
+                                                           int offset, int interleaved) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = blockIdx.x, h = blockIdx.y * 4 + wave;
   if (h >= H) return;
+  // (out may be a: a thread reads both numbers of its pair before it writes them, and no two threads share a number)
   const float* src = a + (size_t)m * lda + (size_t)h * n;
   float* dst = out + (size_t)m * ldo + (size_t)h * n;
-  const int pos = positions[m];
+  const int pos = half > 0 ? positions[m] : 0;
   for (int i = lane; i < half; i += 64) {
     float sn, cs;
     ro_sincos(pos, freq[i], sign, &sn, &cs);
-    const float u = src[i], v = src[i + half];
-    dst[i] = (u * cs - v * sn) * gain;
-    dst[i + half] = (v * cs + u * sn) * gain;
+    const int iu = offset + (interleaved ? 2 * i : i), iv = offset + (interleaved ? 2 * i + 1 : i + half);
+    const float u = src[iu], v = src[iv];
+    dst[iu] = (u * cs - v * sn) * gain;
+    dst[iv] = (v * cs + u * sn) * gain;
   }
-  for (int d = 2 * half + lane; d < n; d += 64) dst[d] = src[d] * gain;
+  if (src != dst || gain != 1.f) {
+    for (int d = lane; d < offset; d += 64) dst[d] = src[d] * gain;
+    for (int d = offset + 2 * half + lane; d < n; d += 64) dst[d] = src[d] * gain;
+  }
 }
 
 int hy_rotate_heads(const float* a, int lda, const int32_t* positions, const double* freq, int half, int M, int H, int n,
-                    float sign, float gain, float* out, int ldo, hipStream_t s) {
+                    float sign, float gain, float* out, int ldo, int offset, int interleaved, hipStream_t s) {
   if (M < 0 || H < 1 || n < 1 || lda < H * n || ldo < H * n) return -1;
-  if (half < 0 || 2 * half > n || (half > 0 && !freq)) return -2;
+  if (half < 0 || offset < 0 || offset + 2 * half > n || (half > 0 && !freq)) return -2;
   if (M == 0) return 0;
   if ((H + 3) / 4 > 65535) return -4;
-  rotate_heads_kernel<<<dim3(M, (H + 3) / 4), 256, 0, s>>>(a, lda, positions, freq, half, H, n, sign, gain, out, ldo);
+  rotate_heads_kernel<<<dim3(M, (H + 3) / 4), 256, 0, s>>>(a, lda, positions, freq, half, H, n, sign, gain, out, ldo,
+                                                             offset, interleaved);
   JLA_CHECK_LAUNCH();
   return 0;
 }
