@@ -1,0 +1,743 @@
+"""Zifisun through the framework (model, cache, stepper, engine) against the plain float64 oracle
+(tests/oracle_zifisun.py), on the CPU op path and, marked gpu, on the HIP kernels. Small configurations built here: sizes
+that are multiples of nothing, 1 / 2 / 4 residual streams and a plain residual, a looped run of layers, layers without a
+feed-forward, windows with and without kept first keys and no window at all, rotary over part of the rotated key part,
+routers with and without groups, identity experts, a selection bias and a shared expert, top-1 routing."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_zifisun as oz
+from jax_llama_amd.config import NormedAttentionSpec, RotaryLatentSpec, ZifisunConfig
+from jax_llama_amd.models.kv_cache import HybridCache
+from jax_llama_amd.models.mixers import (GroupedMoE, HyperBlock, NormedGatedAttention, RotaryLatentAttention,
+                                         StepContext)
+from jax_llama_amd.models.zifisun import ZifisunForCausalLM, random_state_dict
+from jax_llama_amd.ops import hybrid as hy
+from jax_llama_amd.runtime.engine import GenerationConfig
+from jax_llama_amd.runtime.stepper import SequenceStepper
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+def _lat(heads, dim, rot_dim, vdim, rank, q_rank, scale, window=None, keep_first=None, rot_dims=None, base=10000.0):
+    out = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=rank, q_rank=q_rank, scale=scale,
+               rot={"base": base, "dims": rot_dim if rot_dims is None else rot_dims})
+    if window:
+        out["mask"] = {"size": window}
+        if keep_first:
+            out["mask"]["keep_first"] = keep_first
+    return out
+
+
+def _att(heads, kv_heads, dim, vdim, scale, window=None, keep_first=None):
+    out = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if window:
+        out["mask"] = {"size": window}
+        if keep_first:
+            out["mask"]["keep_first"] = keep_first
+    return out
+
+
+def _moe(experts, top, ff, identity=0, groups=None, shared=0):
+    router = {"experts": experts, "top": top}
+    if identity:
+        router["identity"] = identity
+    if groups:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    out = {"kind": "moe", "expert": {"ff": ff}, "router": router}
+    if shared:
+        out["shared"] = {"ff": shared}
+    return out
+
+
+def cfg_full():
+    """Three streams, layers 1-2 run twice, both mixers, windows shorter than the test prompts."""
+    return {"architecture": "Zifisun", "vocab": 67, "width": 40, "norm": {"eps": 1e-5}, "streams": 3,
+            "loop": {"start": 1, "stop": 3, "times": 2},
+            "layers": [
+                {"type": "latent_attention", "mixer": _lat(3, 16, 8, 24, 20, 28, 0.2, window=9),
+                 "mlp": _moe(6, 3, 24, identity=2, groups=(4, 3), shared=40)},
+                {"type": "attention", "mixer": _att(4, 2, 12, 20, 0.3, window=13, keep_first=4), "mlp": _moe(5, 2, 16, identity=1)},
+                {"type": "latent_attention", "mixer": _lat(2, 8, 12, 8, 36, 16, 0.25, window=21, keep_first=3, rot_dims=6,
+                                                            base=500.0), "mlp": None},
+                {"type": "attention", "mixer": _att(6, 6, 8, 8, 0.35), "mlp": _moe(8, 4, 8, groups=(2, 1), shared=24)},
+            ]}
+
+
+def cfg_bare():
+    """No streams entry (a plain residual), no loop, one head, one expert, top 1, no correction-free shortcuts."""
+    return {"architecture": "Zifisun", "vocab": 37, "width": 24, "norm": {"eps": 1e-6},
+            "layers": [
+                {"type": "attention", "mixer": _att(1, 1, 8, 40, 1.0, window=5, keep_first=1), "mlp": _moe(1, 1, 16)},
+                {"type": "latent_attention", "mixer": _lat(1, 8, 2, 8, 8, 8, 0.35), "mlp": _moe(3, 1, 8, identity=3)},
+            ]}
+
+
+def cfg_streams(n):
+    c = cfg_full()
+    c["streams"] = n
+    c["loop"] = {"start": 0, "stop": 2, "times": 3}
+    return c
+
+
+def build(cfg, device, dtype=F32, seed=0, edit=None):
+    config = ZifisunConfig.from_dict(cfg)
+    sd = random_state_dict(config, seed=seed)
+    for k in list(sd):
+        if k.endswith("mlp.router"):  # clearly separated scores: no near-ties in the choice
+            sd[k] = (sd[k].float() * 3.0).to(BF16)
+        if k.endswith("mlp.correction"):  # a selection bias large enough to change choices
+            sd[k] = (sd[k].float() * 4.0).to(BF16)
+    if edit:
+        edit(sd)
+    model = ZifisunForCausalLM(config, device=device, dtype=dtype, _do_init=False).load_state_dict(sd)
+    return model, sd
+
+
+def toks(n, vocab, seed=1):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def err(got, ref):
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    d = got - ref
+    return float(np.sqrt(np.mean(d * d)) / np.sqrt(np.mean(ref * ref)))
+
+
+def tol(device, dtype=F32):
+    return 3e-2 if dtype == BF16 else 2e-5
+
+
+def run_portions(model, tokens, portions, rid="r", stepper=None, max_tokens=None):
+    """Logits of every position through the stepper, the prompt cut into ``portions``."""
+    st = stepper or SequenceStepper(model, max_tokens or len(tokens))
+    out, at = [], 0
+    for n in portions:
+        out.append(st.feed(rid, tokens[at:at + n], list(range(n))).float().cpu())
+        at += n
+    assert at == len(tokens)
+    st.end(rid)
+    return torch.cat(out).numpy()
+
+
+# ---------------------------------------------------------------------------------------------- configuration
+def test_config_round_trip():
+    c = ZifisunConfig.from_dict(cfg_full())
+    assert ZifisunConfig.from_dict(c.to_dict()) == c
+    assert c.layer_runs() == [0, 1, 2, 1, 2, 3] and c.num_hidden_layers == 6 and c.streams == 3
+    assert isinstance(c.layers[0].mixer, RotaryLatentSpec) and isinstance(c.layers[1].mixer, NormedAttentionSpec)
+    assert (c.layers[0].mixer.window, c.layers[0].mixer.keep_first) == (9, 0)
+    assert (c.layers[1].mixer.window, c.layers[1].mixer.keep_first) == (13, 4) and c.layers[3].mixer.window == 0
+    assert c.layers[2].mixer.rot_dims == 6 and c.layers[2].mixer.rot_dim == 12 and c.layers[2].mlp is None
+    f = c.layers[0].mlp
+    assert (f.experts, f.identity, f.top, f.groups, f.keep_groups, f.shared_ff) == (6, 2, 3, 4, 3, 40)
+    assert c.layers[1].mlp.groups == 1 and c.layers[1].mlp.shared_ff == 0
+    b = ZifisunConfig.from_dict(cfg_bare())
+    assert b.streams == 0 and b.layer_runs() == [0, 1] and ZifisunConfig.from_dict(b.to_dict()) == b
+    for breaker in (lambda d: d["layers"][0]["mlp"]["router"].update(top=7),          # more choices than the kept groups hold
+                    lambda d: d["layers"][0]["mlp"]["router"]["groups"].update(count=3),  # 8 experts in 3 groups
+                    lambda d: d["layers"][1].update(type="delta"),
+                    lambda d: d["loop"].update(stop=9),
+                    lambda d: d["layers"][2]["mixer"]["rot"].update(dims=7)):
+        bad = cfg_full()
+        breaker(bad)
+        with pytest.raises(ValueError):
+            ZifisunConfig.from_dict(bad)
+
+
+# ---------------------------------------------------------------------------------------------- mechanisms alone
+def _latent_weights(g, mc, d):
+    r = lambda *s, sc: torch.randn(*s, generator=g) * sc  # noqa: E731
+    nh, kd, rank = mc["heads"], mc["dim"] + mc["rot_dim"], mc["kv_rank"]
+    return {"m.dq": r(mc["q_rank"], d, sc=0.4), "m.dq.norm": torch.rand(mc["q_rank"], generator=g) + 0.5,
+            "m.uq": r(nh * kd, mc["q_rank"], sc=0.4), "m.dkv": r(rank + mc["rot_dim"], d, sc=0.4),
+            "m.dkv.norm": torch.rand(rank, generator=g) + 0.5, "m.uk": r(nh * mc["dim"], rank, sc=0.4),
+            "m.uv": r(nh * mc["vdim"], rank, sc=0.4), "m.g": r(nh, d, sc=0.5), "m.o": r(d, nh * mc["vdim"], sc=0.2)}
+
+
+def _run_latent(w, mc, h, eps, device, portions, dtype=F32, form=None):
+    """The framework's latent attention on hand-made inputs ``h`` in portions, through the mixer block and the cache."""
+    sp = RotaryLatentSpec.from_dict(mc)
+    t = h.shape[0]
+    cache = HybridCache([("latent", sp.kv_rank + sp.rot_dim)], 1, t, device, dtype)
+    w_uk = w["m.uk"].reshape(sp.heads, sp.dim, sp.kv_rank).to(device, dtype)
+    w_uv = w["m.uv"].reshape(sp.heads, sp.vdim, sp.kv_rank).contiguous().to(device, dtype)
+    freq = hy.rotary_freqs(sp.rot_base, sp.rot_dims, device) if sp.rot_dims else None
+    mixer = RotaryLatentAttention(0, sp, eps, torch.cat([w["m.dq"], w["m.dkv"], w["m.g"]]).to(device, dtype),
+                                  w["m.dq.norm"].to(device), w["m.uq"].to(device, dtype), w["m.dkv.norm"].to(device),
+                                  w_uk, w_uv, freq, w["m.o"].to(device, dtype))
+    if form is not None:  # pin the form: in the latent space, or expanded for portions of two tokens and more
+        mixer.expands = lambda s, n, bf16: form == "expanded"
+    outs, s0 = [], 0
+    for s in portions:
+        ids = torch.zeros(s, dtype=torch.int32, device=device)
+        pos = torch.arange(s0, s0 + s, dtype=torch.int32, device=device)
+        outs.append(mixer(h[s0:s0 + s].to(device), StepContext(ids, pos, 1, s, cache, s0)).cpu())
+        s0 += s
+    assert s0 == t
+    return torch.cat(outs).numpy()
+
+
+def _attn_weights(g, mc, d):
+    r = lambda *s, sc: torch.randn(*s, generator=g) * sc  # noqa: E731
+    nh, ng = mc["heads"], mc["kv_heads"]
+    return {"m.q": r(nh * mc["dim"], d, sc=0.4), "m.k": r(ng * mc["dim"], d, sc=0.4), "m.v": r(ng * mc["vdim"], d, sc=0.4),
+            "m.q.norm": torch.rand(mc["dim"], generator=g) + 0.5, "m.k.norm": torch.rand(mc["dim"], generator=g) + 0.5,
+            "m.g": r(nh, d, sc=0.5), "m.o": r(d, nh * mc["vdim"], sc=0.2)}
+
+
+def _run_attn(w, mc, h, eps, device, portions, dtype=F32):
+    sp = NormedAttentionSpec.from_dict(mc)
+    t = h.shape[0]
+    cache = HybridCache([("kv", sp.kv_heads, sp.dim, sp.vdim)], 1, t, device, dtype)
+    mixer = NormedGatedAttention(0, sp, eps, torch.cat([w["m.q"], w["m.k"], w["m.v"], w["m.g"]]).to(device, dtype),
+                                 w["m.q.norm"].to(device), w["m.k.norm"].to(device), True, w["m.o"].to(device, dtype))
+    outs, s0 = [], 0
+    for s in portions:
+        ids = torch.zeros(s, dtype=torch.int32, device=device)
+        pos = torch.arange(s0, s0 + s, dtype=torch.int32, device=device)
+        outs.append(mixer(h[s0:s0 + s].to(device), StepContext(ids, pos, 1, s, cache, s0)).cpu())
+        s0 += s
+    assert s0 == t
+    return torch.cat(outs).numpy()
+
+
+LATENT_SHAPES = [  # heads, dim, rot_dim, vdim, rank, q_rank, window, keep_first, rot_dims
+    (3, 16, 8, 24, 20, 28, 9, 0, None), (1, 8, 2, 72, 56, 8, 0, 0, None), (12, 8, 4, 8, 24, 16, 17, 5, 2),
+    (70, 8, 2, 4, 16, 8, 64, 0, None), (2, 24, 16, 40, 64, 32, 1, 0, None), (2, 16, 16, 16, 200, 24, 23, 23, None),
+    (2, 16, 6, 16, 500, 24, 30, 2, 0)]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("heads,dim,rot_dim,vdim,rank,q_rank,window,keep,rot_dims", LATENT_SHAPES)
+def test_latent_attention_mechanism(device, heads, dim, rot_dim, vdim, rank, q_rank, window, keep, rot_dims):
+    """One latent-attention sublayer against the oracle (which materialises every head's keys and values), in portions
+    that include single tokens and pairs, both forms; windows of one key, of a 64-key chunk, wider than the kept prefix and
+    equal to it; no rotation at all and rotation over part of the rotated numbers."""
+    mc = _lat(heads, dim, rot_dim, vdim, rank, q_rank, 0.31, window, keep, rot_dims, base=300.0)
+    t, d, eps = 71, 48, 1e-6
+    g = torch.Generator().manual_seed(3)
+    w = _latent_weights(g, mc, d)
+    h = torch.randn(t, d, generator=g)
+    ref = oz.latent_attention(w, "m.", mc, h.double().numpy(), eps)
+    for form in ("latent", "expanded", None):
+        got = _run_latent(w, mc, h, eps, device, [11, 1, 2, 29, 1, 1, 20, 6], form=form)
+        assert err(got, ref) < 2e-5, form
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,window,keep", [(4, 2, 12, 20, 13, 4), (1, 1, 8, 72, 0, 0),
+                                                                 (6, 6, 16, 8, 1, 0), (70, 35, 8, 4, 64, 64),
+                                                                 (8, 1, 24, 40, 30, 70), (2, 2, 64, 64, 19, 3)])
+def test_normed_attention_mechanism(device, heads, kv_heads, dim, vdim, window, keep):
+    """One attention sublayer against the oracle: weighted q / k norms, grouped heads, windows with kept first keys
+    (kept prefix shorter than, equal to and longer than the window), gates."""
+    mc = _att(heads, kv_heads, dim, vdim, 0.4, window, keep)
+    t, d, eps = 90, 48, 1e-6
+    g = torch.Generator().manual_seed(5)
+    w = _attn_weights(g, mc, d)
+    h = torch.randn(t, d, generator=g)
+    ref = oz.attention(w, "m.", mc, h.double().numpy(), eps)
+    got = _run_attn(w, mc, h, eps, device, [11, 1, 2, 38, 1, 1, 30, 6])
+    assert err(got, ref) < 2e-5
+    assert err(_run_attn(w, mc, h, eps, device, [1] * t), ref) < 2e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_at_the_mfma_head_sizes(device, dtype):
+    """Head sizes the flash prefill kernel takes (bf16), with windows and kept keys that end inside its 32-key tiles and
+    portions that start at unaligned slots; the latent attention's expanded form at a key width of 64 + 64."""
+    t, d, eps = 300, 96, 1e-6
+    g = torch.Generator().manual_seed(9)
+    h = torch.randn(t, d, generator=g).to(BF16).float()
+    lim = 3e-2 if dtype == BF16 else 2e-5
+    for dim, vdim, window, keep in [(64, 128, 45, 0), (128, 64, 70, 37), (64, 64, 33, 100), (128, 128, 0, 0)]:
+        mc = _att(4, 2, dim, vdim, dim ** -0.5 * 4.0, window, keep)
+        w = {k: v.to(BF16).float() for k, v in _attn_weights(g, mc, d).items()}
+        ref = oz.attention(w, "m.", mc, h.double().numpy(), eps)
+        got = _run_attn(w, mc, h, eps, device, [100, 2, 147, 1, 50], dtype)
+        assert err(got, ref) < lim, (dim, vdim, window, keep)
+    mc = _lat(3, 64, 64, 64, 96, 48, 0.1, 50, 9, base=1e4)
+    w = {k: v.to(BF16).float() for k, v in _latent_weights(g, mc, d).items()}
+    ref = oz.latent_attention(w, "m.", mc, h.double().numpy(), eps)
+    for form in ("latent", "expanded"):
+        assert err(_run_latent(w, mc, h, eps, device, [100, 2, 147, 1, 50], dtype, form), ref) < lim, form
+
+
+def _point_at(wq, key):
+    """An input whose projection by ``wq [n, d]`` (n <= d) is ``key``: the least-squares solution."""
+    return np.linalg.lstsq(wq, key, rcond=None)[0]
+
+
+def _edge_targets(i, window, keep):
+    """Keys whose visibility from query ``i`` hangs on one constant: the oldest key inside the window, the newest one
+    outside it, the last kept key, the first key that is not kept."""
+    return {"window_in": i - window + 1, "window_out": i - window, "first_in": keep - 1, "first_out": keep}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_keys_at_the_edges_decide(device, dtype):
+    """Eight late queries, four inside a portion and four decoded alone, are solved so that head 0 points at one key
+    each: the oldest key inside its window, the newest outside it, the last kept first key and the first one not kept
+    (300 positions back). Where the key is visible it takes nearly all of the head's weight; where it is hidden the head
+    falls back on the others. A window or a kept prefix that is one off moves those rows by far more than the tolerance."""
+    heads, dim, vdim, d, t, eps, window, keep = 2, 32, 24, 48, 333, 1e-6, 37, 11
+    mc = _att(heads, 1, dim, vdim, 1.5, window, keep)
+    g = torch.Generator().manual_seed(7)
+    w = {k: v.to(BF16).float() for k, v in _attn_weights(g, mc, d).items()}
+    w["m.q.norm"] = torch.ones(dim)
+    w["m.k.norm"] = torch.ones(dim)
+    w["m.g"][0] = 0.0  # head 0's gate stays at one half whatever the solved inputs are
+    h = (torch.randn(t, d, generator=g) * 0.3).to(BF16).float()
+    hn = h.double().numpy()
+    k_raw = hn @ w["m.k"].double().numpy().T  # one key head
+    rows = {}
+    for base in (296, 329):  # inside the portion 290 .. 326, and among the tokens decoded alone
+        for n, (kind, j) in enumerate(_edge_targets(0, window, keep).items()):
+            i = base + n
+            j = _edge_targets(i, window, keep)[kind]
+            h[i] = torch.tensor(_point_at(w["m.q"].double().numpy()[:dim], k_raw[j]), dtype=F32).to(BF16).float()
+            rows[i] = (kind, j)
+    hn = h.double().numpy()
+    ref, pw = oz.attention(w, "m.", mc, hn, eps, return_weights=True)
+    for i, (kind, j) in rows.items():
+        if kind.endswith("_in"):
+            assert pw[0, i, j] > 0.9, (i, kind, pw[0, i, j])
+        else:
+            assert pw[0, i, j] == 0.0
+    lim = 3e-2 if dtype == BF16 else 2e-5
+    got = _run_attn(w, mc, h, eps, device, [290, 37] + [1] * 6, dtype)
+    assert err(got, ref) < lim
+    for i in rows:
+        assert err(got[i], ref[i]) < 2 * lim, (i, rows[i])
+    # the same rows under a window or a kept prefix that is one off
+    for kind, change in (("window_in", dict(size=window - 1)), ("window_out", dict(size=window + 1)),
+                         ("first_in", dict(keep_first=keep - 1)), ("first_out", dict(keep_first=keep + 1))):
+        off_mc = dict(mc, mask=dict(mc["mask"], **change))
+        off = oz.attention(w, "m.", off_mc, hn, eps)
+        for i, (k2, _) in rows.items():
+            if k2 == kind:
+                assert err(off[i], ref[i]) > 0.2, (i, kind)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_latent_keys_at_the_edges_decide(device, dtype):
+    """The same construction for the latent attention (the query is solved through its latent and up projection, the
+    key is the plain part of head 0): window edges and a kept prefix, inside a portion and decoded alone, both forms."""
+    heads, dim, rot, vdim, rank, q_rank, d, t, eps, window, keep = 2, 32, 4, 24, 40, 36, 48, 333, 1e-6, 41, 7
+    mc = _lat(heads, dim, rot, vdim, rank, q_rank, 0.8, window, keep, base=100.0)
+    g = torch.Generator().manual_seed(12)
+    w = {k: v.to(BF16).float() for k, v in _latent_weights(g, mc, d).items()}
+    w["m.dq.norm"] = torch.ones(q_rank)
+    w["m.g"][0] = 0.0  # head 0's gate stays at one half whatever the solved inputs are
+    h = (torch.randn(t, d, generator=g) * 0.3).to(BF16).float()
+    hn = h.double().numpy()
+    c = oz.rms(hn @ w["m.dkv"].double().numpy()[:rank].T, eps) * w["m.dkv.norm"].double().numpy()
+    k_plain = c @ w["m.uk"].double().numpy()[:dim].T  # head 0's plain keys
+    uq0 = w["m.uq"].double().numpy()[:dim]            # head 0's plain query rows
+    rows = {}
+    for base in (296, 329):
+        for n, kind in enumerate(("window_in", "window_out", "first_in", "first_out")):
+            i = base + n
+            j = _edge_targets(i, window, keep)[kind]
+            cq = _point_at(uq0, k_plain[j])
+            h[i] = torch.tensor(_point_at(w["m.dq"].double().numpy(), cq), dtype=F32).to(BF16).float()
+            rows[i] = (kind, j)
+    hn = h.double().numpy()
+    ref, pw = oz.latent_attention(w, "m.", mc, hn, eps, return_weights=True)
+    for i, (kind, j) in rows.items():
+        if kind.endswith("_in"):
+            assert pw[0, i, j] > 0.9, (i, kind, pw[0, i, j])
+        else:
+            assert pw[0, i, j] == 0.0
+    lim = 3e-2 if dtype == BF16 else 2e-5
+    for form in ("latent", "expanded"):
+        got = _run_latent(w, mc, h, eps, device, [290, 37] + [1] * 6, dtype, form)
+        assert err(got, ref) < lim, form
+        for i in rows:
+            assert err(got[i], ref[i]) < 2 * lim, (form, i, rows[i])
+    for kind, change in (("window_in", dict(size=window - 1)), ("window_out", dict(size=window + 1)),
+                         ("first_in", dict(keep_first=keep - 1)), ("first_out", dict(keep_first=keep + 1))):
+        off = oz.latent_attention(w, "m.", dict(mc, mask=dict(mc["mask"], **change)), hn, eps)
+        for i, (k2, _) in rows.items():
+            if k2 == kind:
+                assert err(off[i], ref[i]) > 0.2, (i, kind)
+    # a rotation that is one position off (queries turned as if they sat one slot later) moves every row
+    shifted = oz.latent_attention(w, "m.", mc, hn, eps, pos=np.arange(t) * 1.0 + (np.arange(t) % 2))
+    assert err(shifted, ref) > 0.05
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_interleaved_rotation_and_latent_prep(device):
+    """The two position-dependent kernels alone: the rotated tail of each query head in place (pairs 2i, 2i + 1, from an
+    offset, over part of the tail), and the prep that norms both latents and caches the rotated shared key part."""
+    g = torch.Generator().manual_seed(2)
+    m, heads, dim, rot, dims = 9, 5, 6, 10, 6
+    x = torch.randn(m, heads * (dim + rot), generator=g)
+    pos = torch.tensor([0, 1, 2, 3, 1000, 4097, 5, 77, 31], dtype=torch.int32)
+    freq = hy.rotary_freqs(1e4, dims, device)
+    ref = x.double().numpy().reshape(m, heads, dim + rot).copy()
+    ref[..., dim:] = oz.rotate_pairs(ref[..., dim:], pos.numpy(), 1e4, dims)
+    xd = x.to(device).clone()
+    out = hy.rotate_heads(xd, pos.to(device), freq, heads, out=xd, offset=dim, interleaved=True)
+    assert out is xd and err(xd.cpu().numpy().reshape(m, heads, dim + rot), ref) < 1e-6
+    b, s, q_rank, rank, eps = 2, 4, 7, 5, 1e-5
+    proj = torch.randn(b * s, q_rank + rank + rot + 3, generator=g)
+    qw, cw = torch.rand(q_rank, generator=g) + 0.5, torch.rand(rank, generator=g) + 0.5
+    pos = torch.arange(3, 3 + s, dtype=torch.int32).repeat(b)
+    cache = torch.zeros(b, 1, 9, rank + rot, device=device)
+    cq = hy.latent_rope_prep(proj.to(device), 0, qw.to(device), q_rank, cw.to(device), freq, pos.to(device), 3, b, s, cache,
+                             eps)
+    pn = proj.double().numpy()
+    assert err(cq.cpu().numpy(), oz.rms(pn[:, :q_rank], eps) * qw.double().numpy()) < 1e-6
+    want = np.concatenate([oz.rms(pn[:, q_rank:q_rank + rank], eps) * cw.double().numpy(),
+                           oz.rotate_pairs(pn[:, q_rank + rank:q_rank + rank + rot], pos.numpy(), 1e4, dims)], -1)
+    assert err(cache[:, 0, 3:3 + s].reshape(b * s, -1).cpu().numpy(), want) < 1e-6
+    assert float(cache[:, 0, :3].abs().max()) == 0.0 and float(cache[:, 0, 3 + s:].abs().max()) == 0.0
+
+
+def _moe_weights(g, d, fc, scale=1.0):
+    r = lambda *s, sc: torch.randn(*s, generator=g) * sc  # noqa: E731
+    rc = fc["router"]
+    total = rc["experts"] + rc.get("identity", 0)
+    w = {"f.router": r(total, d, sc=scale), "f.correction": r(total, sc=0.1)}
+    for e in range(rc["experts"]):
+        w.update({f"f.e{e}.up": r(fc["expert"]["ff"], d, sc=0.4), f"f.e{e}.down": r(d, fc["expert"]["ff"], sc=0.3)})
+    if fc.get("shared"):
+        w.update({"f.shared.up": r(fc["shared"]["ff"], d, sc=0.4), "f.shared.down": r(d, fc["shared"]["ff"], sc=0.3)})
+    return w
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("m,experts,identity,top,groups,shared", [
+    (1, 4, 0, 2, None, 24), (2, 6, 2, 3, (4, 3), 0), (3, 6, 2, 4, (4, 2), 40), (40, 5, 1, 2, (3, 2), 40),
+    (70, 1, 0, 1, None, 0), (9, 60, 10, 4, (7, 3), 16), (300, 6, 3, 1, (3, 1), 8), (17, 2, 6, 3, (2, 2), 0)])
+def test_grouped_mixture(device, m, experts, identity, top, groups, shared):
+    """Router (softmax scores, selection bias, groups, identity experts), squared-ReLU experts weighted on their output,
+    shared expert, summed by the stream update; row counts of the per-row GEMV, the expert-grouped GEMV and the tiles."""
+    d = 40
+    fc = _moe(experts, top, 24, identity, groups, shared)
+    g = torch.Generator().manual_seed(5)
+    w = _moe_weights(g, d, fc)
+    x = torch.randn(m, d, generator=g)
+    xn = x.double().numpy()
+    chosen, weight = oz.route(w, "f.", fc, xn)
+    if identity and m >= 9:
+        assert (chosen >= experts).any() and (chosen < experts).any()  # both kinds of expert are used
+    ref = oz.moe(w, "f.", fc, xn)
+    moe = GroupedMoE(experts, identity, top, groups[0] if groups else 1, groups[1] if groups else 1,
+                     w["f.router"].to(device), w["f.correction"].to(device),
+                     torch.stack([w[f"f.e{e}.up"] for e in range(experts)]).to(device),
+                     torch.stack([w[f"f.e{e}.down"] for e in range(experts)]).to(device),
+                     w["f.shared.up"].to(device) if shared else None, w["f.shared.down"].to(device) if shared else None)
+    f = moe(x.to(device), None)
+    assert f.nsum == top and f.y.shape == (m * top, d)
+    assert np.array_equal(np.sort(f.row_expert.reshape(m, top).cpu().numpy(), -1), np.sort(chosen, -1))
+    xs = torch.zeros(1, m, d, device=device)
+    one = torch.ones(1, device=device)
+    u = hy.hc_update_(xs, one.reshape(1, 1), one, f.y, f.nsum, f.row_w, f.row_expert, f.n_real, f.ident, f.extra,
+                      next_in=one)
+    assert err(xs[0].cpu().numpy(), ref) < 2e-5 and torch.equal(u, xs[0])
+    # the router's own record: experts by descending choice score, weights = the scores without the bias
+    ex, wt = hy.route_grouped(hy.linear(x, w["f.router"]), w["f.correction"], top, groups[0] if groups else 1,
+                              groups[1] if groups else 1)
+    assert np.array_equal(ex.reshape(m, top).numpy(), chosen) and err(wt.reshape(m, top).numpy(), weight) < 1e-5
+
+
+def test_group_limit_and_selection_bias_change_the_choice():
+    """The pieces of the router that random weights rarely separate: an expert with the largest score in a group that
+    is not kept is not chosen; the bias moves the choice but not the weight; hidden experts count as minus infinity
+    even where every visible choice score is negative."""
+    z = torch.tensor([[4.0, 0.0, 0.1, 0.2, 3.0, 2.9, 0.0, 0.0]])  # groups of 2: {4.0, 0}, {.1, .2}, {3, 2.9}, {0, 0}
+    ex, wt = hy.route_grouped(z, None, 2, groups=4, keep=1)
+    assert ex.tolist() == [0, 1]                                     # group 0 only, although 3.0 > 0.0
+    ex, wt = hy.route_grouped(z, None, 2, groups=4, keep=2)
+    assert ex.tolist() == [0, 4] and abs(float(wt[0]) - float(torch.softmax(z, -1)[0, 0])) < 1e-7
+    corr = torch.tensor([-5.0, -5.0, -4.0, -4.5, -9.0, -9.0, -9.0, -9.0])  # all choice scores negative
+    ex, wt = hy.route_grouped(z, corr, 2, groups=4, keep=1)
+    assert ex.tolist() == [2, 3] and abs(float(wt[0]) - float(torch.softmax(z, -1)[0, 2])) < 1e-7
+    w = {"f.router": torch.eye(8), "f.correction": corr}
+    chosen, weight = oz.route(w, "f.", _moe(8, 2, 4, groups=(4, 1)), z.double().numpy())
+    assert chosen.tolist() == [[2, 3]] and abs(weight[0, 0] - float(wt[0])) < 1e-6
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("streams,m,d", [(1, 3, 40), (2, 1, 24), (3, 70, 40), (4, 5, 300), (8, 2, 1030)])
+def test_stream_update(device, streams, m, d):
+    """The hyper-connection kernels alone: the read (a weighted sum of the streams) and the write (all streams at once
+    from the old ones, the mixing matrix indexed [from, to], which a transposed matrix would get wrong)."""
+    g = torch.Generator().manual_seed(6)
+    xs = torch.randn(streams, m, d, generator=g)
+    a, c, nxt = (torch.randn(streams, generator=g) for _ in range(3))
+    mix = torch.randn(streams, streams, generator=g)
+    y = torch.randn(m, d, generator=g)
+    assert err(hy.hc_in(xs.to(device), a.to(device)).cpu().numpy(), np.einsum("s,smd->md", a.numpy(), xs.numpy())) < 1e-6
+    want = np.einsum("st,smd->tmd", mix.double().numpy(), xs.double().numpy()) + \
+        c.double().numpy()[:, None, None] * y.double().numpy()[None]
+    xd = xs.to(device).clone()
+    u = hy.hc_update_(xd, mix.to(device), c.to(device), y.to(device), next_in=nxt.to(device))
+    assert err(xd.cpu().numpy(), want) < 1e-6
+    assert err(u.cpu().numpy(), np.einsum("t,tmd->md", nxt.double().numpy(), want)) < 1e-5
+    if streams > 1:
+        wrong = np.einsum("ts,smd->tmd", mix.double().numpy(), xs.double().numpy())
+        assert err(wrong + c.double().numpy()[:, None, None] * y.double().numpy()[None], want) > 0.1
+
+
+# ---------------------------------------------------------------------------------------------- whole model
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cfg", [cfg_full, cfg_bare, lambda: cfg_streams(1), lambda: cfg_streams(2), lambda: cfg_streams(4)])
+def test_prompt_logits_and_residual_stream(device, cfg):
+    model, sd = build(cfg(), device)
+    t = toks(45, model.config.vocab_size)
+    ref, ref_hidden = oz.forward(cfg(), sd, t)
+    ids = torch.tensor([t], dtype=torch.int32)
+    out = model(ids, output_hidden_states=True)
+    assert len(out.hidden_states) == len(ref_hidden) == len(model.config.layer_runs())
+    for i, hs in enumerate(out.hidden_states):
+        assert err(hs[0].cpu().numpy(), ref_hidden[i]) < tol(device), f"layer run {i}"
+    assert err(out.logits[0].cpu().numpy(), ref) < tol(device)
+    assert err(out.logits[0, :3].cpu().numpy(), ref[:3]) < tol(device)  # the first tokens of a sequence
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_bfloat16_serving_format(device):
+    model, sd = build(cfg_full(), device, dtype=BF16)
+    t = toks(40, 67)
+    ref, _ = oz.forward(cfg_full(), sd, t)
+    got = run_portions(model, t, [33] + [1] * 7)
+    assert err(got, ref) < tol(device, BF16)
+    cache = model.init_cache(1, 8)
+    assert len(cache.specs) == 6  # one cache layer per layer run
+    k, v = cache.layer(0)
+    assert k.dtype == BF16 and k is v and k.shape == (1, 1, 8, 20 + 8)  # the latent and the rotated key part
+    k, v = cache.layer(3)  # the second pass of layer 1 has keys of its own
+    assert k.shape == (1, 2, 8, 12) and v.shape == (1, 2, 8, 20) and k.data_ptr() != cache.layer(1)[0].data_ptr()
+    assert cache.nbytes() == model.cache_nbytes(1, 8) == 2 * 8 * (28 + 2 * (2 * 32 + 48) + 6 * 16)
+    assert model.blocks[0].mlp.w_router.dtype == F32 and model.blocks[0].hc1[1].dtype == F32
+    assert model.blocks[1].mixer.w_in is model.blocks[3].mixer.w_in  # the passes of a looped layer share its weights
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cfg", [cfg_full, cfg_bare])
+def test_prefill_against_token_by_token(device, cfg):
+    model, sd = build(cfg(), device)
+    t = toks(34, model.config.vocab_size, seed=2)
+    ref, _ = oz.forward(cfg(), sd, t)
+    whole = run_portions(model, t, [34])
+    single = run_portions(model, t, [1] * 34)
+    assert err(whole, ref) < tol(device) and err(single, ref) < tol(device)
+    assert err(single, whole) < tol(device)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("portions", [[2] * 20, [3, 2, 9, 1, 1, 17, 2, 5], [12, 13, 14, 1], [1, 39], [38, 2]])
+def test_portions_of_any_size(device, portions):
+    model, sd = build(cfg_full(), device, seed=1)
+    t = toks(sum(portions), 67, seed=3)
+    ref, _ = oz.forward(cfg_full(), sd, t)
+    assert err(run_portions(model, t, portions), ref) < tol(device)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding(device):
+    """150 single-token steps after a short prompt: every window passes over decoded tokens, the kept first keys fall
+    far behind, and the unwindowed layer goes past the 64-key chunks and the key splits of the decode kernels."""
+    model, sd = build(cfg_full(), device, seed=2)
+    t = toks(156, 67, seed=4)
+    ref, _ = oz.forward(cfg_full(), sd, t)
+    got = run_portions(model, t, [6] + [1] * 150)
+    e = [err(got[i], ref[i]) for i in range(156)]
+    assert max(e) < tol(device), int(np.argmax(e))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_rows_are_reset_and_reused(device):
+    """A finished request's cache row serves the next request from a clean start; two live requests fed in turns do not
+    touch each other."""
+    model, sd = build(cfg_full(), device)
+    a, b = toks(21, 67, seed=6), toks(17, 67, seed=7)
+    ref_a, _ = oz.forward(cfg_full(), sd, a)
+    ref_b, _ = oz.forward(cfg_full(), sd, b)
+    st = SequenceStepper(model, 32)
+    assert err(run_portions(model, a, [20, 1], "a", st), ref_a) < tol(device)
+    assert st.live() == [] and len(st._free) == 1
+    assert err(run_portions(model, b, [5, 12], "b", st), ref_b) < tol(device)  # the same row again, shorter
+    assert len(st._free) == 1
+    got_a, got_b = [], []
+    for lo in range(0, 21, 3):  # interleaved: two rows live at once
+        got_a.append(st.feed("a", a[lo:lo + 3], list(range(len(a[lo:lo + 3])))).cpu())
+        if lo < 17:
+            got_b.append(st.feed("b", b[lo:lo + 3], list(range(len(b[lo:lo + 3])))).cpu())
+    assert st.live() == ["a", "b"] and st.held("a") == 21 and st.held("b") == 17
+    assert err(torch.cat(got_a).numpy(), ref_a) < tol(device) and err(torch.cat(got_b).numpy(), ref_b) < tol(device)
+    with pytest.raises(ValueError):
+        st.feed("a", toks(12, 67), [])  # more than the row holds
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batch_rows_against_each_alone(device):
+    model, sd = build(cfg_full(), device)
+    rows = [toks(19, 67, seed=8), toks(19, 67, seed=9), toks(19, 67, seed=10)]
+    cache = model.init_cache(3, 24)
+    out = model(torch.tensor(rows, dtype=torch.int32), past_key_values=cache).logits
+    nxt = [[5], [6], [7]]
+    out2 = model(torch.tensor(nxt, dtype=torch.int32), past_key_values=cache).logits  # one decode step of the batch
+    for r in range(3):
+        ref, _ = oz.forward(cfg_full(), sd, rows[r] + nxt[r])
+        assert err(out[r].cpu().numpy(), ref[:19]) < tol(device)
+        assert err(out2[r].cpu().numpy(), ref[19:]) < tol(device)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cfg", [cfg_full, cfg_bare])
+def test_greedy_generation_through_the_engine(device, cfg):
+    """model.generate (prefill + decode steps of the engine, hipGraph replay on the GPU): every generated token is the
+    oracle's argmax of the sequence so far (up to rounding between near-equal logits)."""
+    model, sd = build(cfg(), device)
+    v = model.config.vocab_size
+    prompt = toks(9, v, seed=11)
+    seq = model.generate(torch.tensor([prompt], dtype=torch.int32),
+                         generation_config=GenerationConfig(max_length=40, pad_token_id=0)).sequences[0].cpu().tolist()
+    assert seq[:9] == prompt and len(seq) == 40 and all(0 <= x < v for x in seq)
+    ref, _ = oz.forward(cfg(), sd, seq)
+    for i in range(9, 40):
+        row = ref[i - 1]
+        assert row.max() - row[seq[i]] <= 1e-4 * np.abs(row).max(), i
+    again = model.generate(torch.tensor([prompt], dtype=torch.int32),
+                           generation_config=GenerationConfig(max_length=40, pad_token_id=0)).sequences[0].cpu().tolist()
+    assert again == seq  # the engine's cached cache row starts clean
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_sampled_generation_through_the_engine(device):
+    """The framework's sampler (temperature, top-k, top-p, seeded) on Zifisun logits: reproducible per seed, different
+    across seeds, and every token inside the top-k of the oracle's logits."""
+    model, sd = build(cfg_full(), device)
+    prompt = torch.tensor([toks(7, 67, seed=14)], dtype=torch.int32)
+    gc = dict(max_length=27, pad_token_id=0, do_sample=True, temperature=0.9, top_k=5, top_p=0.95)
+    a = model.generate(prompt, generation_config=GenerationConfig(seed=3, **gc)).sequences[0].cpu().tolist()
+    b = model.generate(prompt, generation_config=GenerationConfig(seed=3, **gc)).sequences[0].cpu().tolist()
+    c = model.generate(prompt, generation_config=GenerationConfig(seed=4, **gc)).sequences[0].cpu().tolist()
+    assert a == b and a != c and all(0 <= x < 67 for x in a + c)
+    ref, _ = oz.forward(cfg_full(), sd, a)
+    for i in range(7, 27):
+        row = ref[i - 1]
+        assert row[a[i]] >= np.sort(row)[-5] - 1e-4 * np.abs(row).max(), i
+
+
+def test_checkpoint_directory_round_trip(tmp_path):
+    from jax_llama_amd.models import registry
+    model, sd = build(cfg_full(), "cpu")
+    model.save_pretrained(str(tmp_path), sd)
+    assert registry.architecture_of(str(tmp_path)) == "zifisun"
+    again = registry.load_model(str(tmp_path), device="cpu", dtype=F32)
+    t = toks(12, 67)
+    ids = torch.tensor([t], dtype=torch.int32)
+    assert torch.equal(again(ids).logits, model(ids).logits)
+    assert registry.supports_dtype("zifisun", F32) and registry.supports_dtype("zifisun", BF16)
+    assert again.weight_bytes() > 0
+    bad = dict(sd)
+    bad["l0.mix.uk"] = bad["l0.mix.uk"][:-1]
+    with pytest.raises(ValueError):
+        ZifisunForCausalLM(model.config, _do_init=False).load_state_dict(bad)
+
+
+def test_trace_runner_program(tmp_path):
+    """bin/trace_run as a user starts it: steps on standard input, logits files, 'done' lines, rows given back."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    model, sd = build(cfg_full(), "cpu")
+    ckpt, out = str(tmp_path / "ckpt"), str(tmp_path / "out")
+    model.save_pretrained(ckpt, sd)
+    a, b = toks(9, 67, seed=12), toks(5, 67, seed=13)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[6:8], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[8:], "want": [0]}], "end": ["a"]},
+             {"step": 3, "entries": [{"id": "b", "tokens": b, "want": [4]}], "end": ["b"]}]
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", ckpt, "--dtype", "float32",
+                        "--out", out, "--max-tokens", "16", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    assert not os.path.exists(os.path.join(out, "1.f32"))
+    ref_a, _ = oz.forward(cfg_full(), sd, a)
+    ref_b, _ = oz.forward(cfg_full(), sd, b)
+    got0 = np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(2, 67)
+    got2 = np.fromfile(os.path.join(out, "2.f32"), dtype="<f4").reshape(1, 67)
+    got3 = np.fromfile(os.path.join(out, "3.f32"), dtype="<f4").reshape(1, 67)
+    assert err(got0, ref_a[[0, 5]]) < 2e-5 and err(got2, ref_a[[8]]) < 2e-5 and err(got3, ref_b[[4]]) < 2e-5
+
+
+def cfg_kernel_shapes():
+    """Head sizes of the MFMA attention kernels (64 / 128) beside plain ones, a cache row wide enough for the shared-latent
+    decode kernel, more heads than a GEMV group, experts with enough rows for the expert-grouped tiles, windows that end
+    inside tiles."""
+    return {"architecture": "Zifisun", "vocab": 300, "width": 192, "norm": {"eps": 1e-6}, "streams": 2,
+            "loop": {"start": 1, "stop": 3, "times": 2},
+            "layers": [{"type": "latent_attention", "mixer": _lat(6, 32, 32, 64, 128, 96, 0.11, window=150),
+                        "mlp": _moe(6, 2, 96, identity=2, groups=(4, 2), shared=64)},
+                       {"type": "attention", "mixer": _att(10, 5, 64, 64, 0.2, window=70, keep_first=37), "mlp": _moe(4, 1, 64)},
+                       {"type": "latent_attention", "mixer": _lat(4, 96, 32, 128, 232, 80, 0.1, window=333, keep_first=5),
+                        "mlp": None},
+                       {"type": "attention", "mixer": _att(4, 1, 128, 64, 0.09), "mlp": _moe(4, 3, 96, identity=4, shared=128)}]}
+
+
+def _router_margins(model, ids, monkeypatch):
+    """Per position, the smallest gap that decides a router's choice over the model's layer runs: between the last
+    chosen and the first rejected choice score among the kept groups, and between the last kept and the first dropped
+    group (read off the framework's own router input while ``model`` runs ``ids``)."""
+    gaps = []
+    grouped = hy.moe_grouped
+
+    def spy(x, z, correction, top, groups, keep, *a, **k):
+        sc = torch.softmax(z.float(), -1)
+        ch = sc + correction.float() if correction is not None else sc
+        gap = torch.full((z.shape[0],), 1.0)
+        if groups > 1:
+            gs = ch.reshape(z.shape[0], groups, -1).max(-1).values.sort(-1, descending=True)
+            if keep < groups:
+                gap = torch.minimum(gap, (gs.values[:, keep - 1] - gs.values[:, keep]).cpu())
+            allowed = torch.zeros(z.shape[0], groups, dtype=torch.bool).scatter_(1, gs.indices[:, :keep].cpu(), True)
+            ch = ch.masked_fill(~allowed.repeat_interleave(z.shape[1] // groups, 1), float("-inf"))
+        cs = ch.sort(-1, descending=True).values
+        if top < z.shape[1]:
+            nxt = cs[:, top]
+            gap = torch.minimum(gap, torch.where(torch.isinf(nxt), gap, (cs[:, top - 1] - nxt).cpu()))
+        gaps.append(gap)
+        return grouped(x, z, correction, top, groups, keep, *a, **k)
+
+    monkeypatch.setattr(hy, "moe_grouped", spy)
+    with torch.no_grad():
+        logits = model(ids).logits[0].numpy()
+    monkeypatch.undo()
+    return logits, torch.stack(gaps).min(0).values.numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_longer_prompts_at_the_kernel_shapes(dtype, monkeypatch):
+    """600 tokens in uneven portions (prompt-sized GEMMs, the flash prefill starting at unaligned slots, decode over
+    several key splits and over windows with kept keys) on the GPU against the framework's fp32 CPU path, which the
+    tests above tie to the oracle. Positions where a router's choice hangs on a gap that bf16 rounding can close are left
+    out of the bf16 comparison (another expert is another function; a handful of 600)."""
+    cfg = cfg_kernel_shapes()
+    ref_model, sd = build(cfg, "cpu", F32)
+    t = toks(600, 300, seed=21)
+    ref, gap = _router_margins(ref_model, torch.tensor([t], dtype=torch.int32), monkeypatch)
+    clear = gap > (0.02 if dtype == BF16 else 1e-4)
+    assert clear.sum() > 400
+    model = ZifisunForCausalLM(ZifisunConfig.from_dict(cfg), device="cuda", dtype=dtype, _do_init=False).load_state_dict(sd)
+    portions = [261, 3, 2, 190, 64, 37] + [1] * 43
+    got = run_portions(model, t, portions)
+    e = np.array([err(got[i], ref[i]) for i in range(600)])
+    assert e[clear].max() < (2e-4 if dtype == F32 else 4e-2), (int(np.argmax(e * clear)), e[clear].max())
+    whole = run_portions(model, t, [600])
+    assert err(whole[clear], got[clear]) < (2e-5 if dtype == F32 else 2e-2)
