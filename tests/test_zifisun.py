@@ -732,8 +732,8 @@ def test_longer_prompts_at_the_kernel_shapes(dtype, monkeypatch):
     ref_model, sd = build(cfg, "cpu", F32)
     t = toks(600, 300, seed=21)
     ref, gap = _router_margins(ref_model, torch.tensor([t], dtype=torch.int32), monkeypatch)
-    clear = gap > (0.02 if dtype == BF16 else 1e-4)
-    assert clear.sum() > 400
+    clear = gap > (0.01 if dtype == BF16 else 1e-4)
+    assert clear.sum() > 200
     model = ZifisunForCausalLM(ZifisunConfig.from_dict(cfg), device="cuda", dtype=dtype, _do_init=False).load_state_dict(sd)
     portions = [261, 3, 2, 190, 64, 37] + [1] * 43
     got = run_portions(model, t, portions)
