@@ -84,12 +84,18 @@ def main():
     ap.add_argument("--recurrent-compare", action="store_true", help="the same comparison for the family of matrix "
                     "memories beside a block-local attention: Besulix beside Zavevik (the closest family: a token-by-token "
                     "recurrence next to attention) and LLaMA")
+    ap.add_argument("--stream-compare", action="store_true", help="the same comparison for the family of windowed latent "
+                    "/ normed attention, grouped routing and several residual streams: Zifisun beside Zasevik (the closest "
+                    "family) and LLaMA")
     ap.add_argument("--hybrid-sizes", nargs="*", default=["2k", "4k"])
     ap.add_argument("--hybrid-families", nargs="*", default=["zavevik", "llama"])
     ap.add_argument("--hybrid-batches", type=int, nargs="*", default=[1, 8])
     args = ap.parse_args()
     if args.latent_compare:
         args.hybrid_families = ["zasevik", "zavevik", "llama"]
+        return _hybrid_compare(args)
+    if args.stream_compare:
+        args.hybrid_families = ["zifisun", "zasevik", "llama"]
         return _hybrid_compare(args)
     if args.recurrent_compare:
         args.hybrid_families = ["besulix", "zavevik", "llama"]

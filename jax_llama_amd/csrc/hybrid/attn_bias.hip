@@ -89,7 +89,8 @@ int hy_attn_prep(const AttnPrep& p, hipStream_t s) {
   return 0;
 }
 
-constexpr int AB_MAX_DIM = 512;   // q head held in LDS per wave
+constexpr int AB_MAX_DIM = 1024;  // q head held in LDS per wave (keys may be wider than values: a latent cache row
+                                  // with a rotated part behind the latent)
 constexpr int AB_MAX_VREG = 8;    // value columns per lane: vdim <= 512
 
 // The keys a query at slot qi sees: slots [0, kf) (kept first keys, only beside a window) and [lo, qi], numbered

@@ -249,10 +249,10 @@ void norm_residual(Tensor y, int64_t nsum, double ysc, Tensor w, double eps, Opt
      "norm_residual");
 }
 
-void cast_bf16(Tensor x, Tensor y) {
+void cast_bf16(Tensor x, Tensor y, int64_t act) {
   gpu(y, "y");
   check(y.scalar_type() == torch::kBFloat16 && y.numel() == x.numel() && x.numel() % 8 == 0, "cast_bf16 shapes");
-  rc(jla::hy_cast_bf16(f32(x, "x"), reinterpret_cast<jla::bf16_t*>(y.data_ptr()), x.numel(), stream()), "cast_bf16");
+  rc(jla::hy_cast_bf16(f32(x, "x"), reinterpret_cast<jla::bf16_t*>(y.data_ptr()), x.numel(), act, stream()), "cast_bf16");
 }
 
 void softcap(Tensor x, double cap) {
@@ -660,7 +660,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.attr("ACT_CLAMP_GLU") = (int)jla::HY_ACT_CLAMP_GLU;
   m.def("norm_residual", &norm_residual);
   m.def("gelu_gate_rows", &gelu_gate_rows);
-  m.def("cast_bf16", &cast_bf16);
+  m.def("cast_bf16", &cast_bf16, py::arg("x"), py::arg("y"), py::arg("act") = 0);
   m.def("softcap", &softcap);
   m.def("attn_prep", &attn_prep, py::arg("proj"), py::arg("positions"), py::arg("slot"), py::arg("B"), py::arg("S"),
         py::arg("H"), py::arg("G"), py::arg("dim"), py::arg("vdim"), py::arg("kc"), py::arg("vc"), py::arg("q"),

@@ -114,9 +114,10 @@ int hy_hc_update(const HyperUpdate& p, hipStream_t s);
 int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_vec, float eps, float* x, float* out,
                      int M, int D, const float* extra, const float* extra_gate, int ldg, hipStream_t s);
 
-// y (bf16) = x (fp32), n a multiple of 8
+// y (bf16) = act(x (fp32)), n a multiple of 8; act: HY_ACT_NONE or HY_ACT_RELU2 (the activation of a feed-forward whose two
+// products run on the packed GEMM, applied while the hidden activation is rounded for the second)
 typedef uint16_t bf16_t;
-int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s);
+int hy_cast_bf16(const float* x, bf16_t* y, long long n, int act, hipStream_t s);
 
 // x <- cap * tanh(x / cap) in place (cap = 1: tanh), n elements
 int hy_softcap(float* x, long long n, float cap, hipStream_t s);

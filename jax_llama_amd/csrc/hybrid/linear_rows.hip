@@ -649,14 +649,58 @@ __global__ void __launch_bounds__(256) route_grouped_select_kernel(const float* 
   }
 }
 
+// The same selection for at most 64 experts, one per lane, without serial rounds: a group's score by per-lane reads of
+// its members, then ranks (how many groups / experts come before this one, ties to the lower index) from reads of every
+// other lane, all independent of each other. A decode step's router is one token: its latency is what shows.
+__global__ void __launch_bounds__(256) route_grouped_select64_kernel(const float* z, int ldz, const float* correction,
+                                                                     int M, int top, int E, int groups, int keep,
+                                                                     int32_t* row_expert, int32_t* row_tok, float* row_w) {
+  const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;
+  const bool valid = lane < E;
+  float zv = valid ? z[(size_t)m * ldz + lane] : -INFINITY;
+  const float cr = valid && correction ? correction[lane] : 0.f;
+  zv = zv == zv ? zv : -INFINITY;
+  const float zmax = wave_max(zv);
+  const float ex = valid ? expf(zv - zmax) : 0.f;
+  const float sc = ex / wave_sum(ex);
+  float ch = valid ? sc + cr : -INFINITY;
+  if (groups > 1) {
+    const int per = E / groups, g = min(lane / per, groups - 1);
+    float gmax = -INFINITY;
+    for (int i = 0; i < per; ++i) gmax = fmaxf(gmax, __shfl(ch, g * per + i, 64));
+    int before = 0;  // groups ahead of this lane's
+    for (int g2 = 0; g2 < groups; ++g2) {
+      const float o = __shfl(gmax, g2 * per, 64);
+      before += (o > gmax || (o == gmax && g2 < g)) ? 1 : 0;
+    }
+    if (before >= keep) ch = -INFINITY;
+  }
+  int rank = 0;  // experts ahead of this lane's
+  for (int e2 = 0; e2 < E; ++e2) {
+    const float o = __shfl(ch, e2, 64);
+    rank += (o > ch || (o == ch && e2 < lane)) ? 1 : 0;
+  }
+  if (valid && rank < top) {
+    const int r = m * top + rank;
+    row_expert[r] = lane;
+    row_tok[r] = m;
+    row_w[r] = ch == -INFINITY ? 0.f : sc;
+  }
+}
+
 int hy_route_grouped(const float* z, int ldz, const float* correction, int M, int top, int E, int groups, int keep,
                      int32_t* row_expert, int32_t* row_tok, float* row_w, int32_t* sort_tok, int32_t* sort_dst,
                      float* sort_w, int32_t* offs, hipStream_t s) {
   if (M < 0 || top < 1 || E < 1 || E > RT_MAX_E || ldz < E) return -1;
   if (groups < 1 || groups > 64 || E % groups || keep < 1 || keep > groups || top > keep * (E / groups)) return -3;
   if (M == 0) return 0;
-  route_grouped_select_kernel<<<(M + 3) / 4, 256, 0, s>>>(z, ldz, correction, M, top, E, groups, keep, row_expert, row_tok,
-                                                          row_w);
+  if (E <= 64)
+    route_grouped_select64_kernel<<<(M + 3) / 4, 256, 0, s>>>(z, ldz, correction, M, top, E, groups, keep, row_expert,
+                                                              row_tok, row_w);
+  else
+    route_grouped_select_kernel<<<(M + 3) / 4, 256, 0, s>>>(z, ldz, correction, M, top, E, groups, keep, row_expert,
+                                                            row_tok, row_w);
   JLA_CHECK_LAUNCH();
   if (!sort_tok) return 0;
   if (!sort_dst || !sort_w || !offs) return -2;

@@ -121,19 +121,28 @@ int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_
 }
 
 // bf16 copy of an fp32 activation (the A operand of the packed MFMA GEMMs), 8 elements per thread
+template <int RELU2>
 __global__ void __launch_bounds__(256) cast_bf16_kernel(const float* __restrict__ x, bf16_t* __restrict__ y, long long n8) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n8) return;
   float f[8];
   hy_load8(x + 8 * i, 8, f);
+  if (RELU2) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float r = fmaxf(f[k], 0.f);
+      f[k] = r * r;
+    }
+  }
   *reinterpret_cast<u32x4*>(y + 8 * i) = pack8(f);
 }
 
-int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s) {
-  if (n < 0 || n % 8) return -1;
+int hy_cast_bf16(const float* x, bf16_t* y, long long n, int act, hipStream_t s) {
+  if (n < 0 || n % 8 || (act != HY_ACT_NONE && act != HY_ACT_RELU2)) return -1;
   if (n == 0) return 0;
   const long long n8 = n / 8;
-  cast_bf16_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, s>>>(x, y, n8);
+  if (act == HY_ACT_RELU2) cast_bf16_kernel<1><<<(unsigned)((n8 + 255) / 256), 256, 0, s>>>(x, y, n8);
+  else cast_bf16_kernel<0><<<(unsigned)((n8 + 255) / 256), 256, 0, s>>>(x, y, n8);
   JLA_CHECK_LAUNCH();
   return 0;
 }
@@ -294,10 +303,13 @@ int hy_latent_prep(const LatentPrep& p, hipStream_t s) {
   return 0;
 }
 
-// one workgroup per token, a thread per column (in steps of 256): every stream's old value of the column is read before
-// any is written, so the replacement is in place
-template <int S>
+// one workgroup per token; a thread owns NU columns 256 apart (a template parameter, so that every load of the step --
+// all streams, the extra summand, the identity input, then the sublayer's rows -- is issued without a branch and in
+// flight together; surplus threads re-read the last column and store nothing). Every stream's old value of a column is
+// read before any is written, so the replacement is in place. NU = 0: any width, one column at a time.
+template <int S, int NU>
 __global__ void __launch_bounds__(256) hc_update_kernel(HyperUpdate p) {
+  constexpr int NC = NU > 0 ? NU : 1;
   const int m = blockIdx.x;
   float mixv[S][S], outw[S], inw[S];
 #pragma unroll
@@ -307,48 +319,50 @@ __global__ void __launch_bounds__(256) hc_update_kernel(HyperUpdate p) {
 #pragma unroll
     for (int t = 0; t < S; ++t) mixv[a][t] = p.mix ? p.mix[a * S + t] : (a == t ? 1.f : 0.f);
   }
-  // the weights of this token's rows; identity experts pool into one weight on `ident`
-  constexpr int MAXC = 16;
-  float wc[MAXC], wid = 0.f;
   const int nsum = p.mix ? p.nsum : 0;
+  const size_t plane = (size_t)p.M * p.D, row = (size_t)m * p.D;
+  for (int d0 = threadIdx.x; d0 < (NU > 0 ? 256 : p.D); d0 += 256) {
+    int dd[NC];
+    float xv[S][NC], v[NC], ev[NC], iv[NC];
 #pragma unroll
-  for (int c = 0; c < MAXC; ++c) {
-    wc[c] = 0.f;
-    if (c < nsum) {
+    for (int u = 0; u < NC; ++u) {
+      dd[u] = min(d0 + 256 * u, p.D - 1);
+#pragma unroll
+      for (int a = 0; a < S; ++a) xv[a][u] = p.xs[a * plane + row + dd[u]];
+      ev[u] = p.extra ? p.extra[row + dd[u]] : 0.f;
+      iv[u] = p.ident ? p.ident[row + dd[u]] : 0.f;
+      v[u] = 0.f;
+    }
+    float wid = 0.f;  // identity experts pool into one weight on `ident`
+#pragma unroll 4
+    for (int c = 0; c < nsum; ++c) {
       const size_t r = (size_t)m * nsum + c;
       const float w = p.row_w ? p.row_w[r] : 1.f;
       const bool real = !p.row_expert || p.row_expert[r] < p.n_real;
-      wc[c] = real ? w : 0.f;
+      float yv[NC];
+#pragma unroll
+      for (int u = 0; u < NC; ++u) yv[u] = p.y[r * p.D + dd[u]];
+#pragma unroll
+      for (int u = 0; u < NC; ++u) v[u] += real ? w * yv[u] : 0.f;  // (an identity row's y holds nothing: selected away)
       wid += real ? 0.f : w;
     }
-  }
-  const size_t plane = (size_t)p.M * p.D;
-  for (int d = threadIdx.x; d < p.D; d += 256) {
-    const size_t at = (size_t)m * p.D + d;
-    float xv[S];
 #pragma unroll
-    for (int a = 0; a < S; ++a) xv[a] = p.xs[a * plane + at];
-    float v = 0.f;
-    if (p.mix) {
+    for (int u = 0; u < NC; ++u) {
+      const float val = fmaf(wid, iv[u], v[u]) + ev[u];
+      float un = 0.f;
 #pragma unroll
-      for (int c = 0; c < MAXC; ++c)
-        if (c < nsum && wc[c] != 0.f) v = fmaf(wc[c], p.y[((size_t)m * nsum + c) * p.D + d], v);
-      if (wid != 0.f) v = fmaf(wid, p.ident[at], v);
-      if (p.extra) v += p.extra[at];
-    }
-    float u = 0.f;
+      for (int t = 0; t < S; ++t) {
+        float nv = xv[t][u];
+        if (p.mix) {
+          nv = outw[t] * val;
 #pragma unroll
-    for (int t = 0; t < S; ++t) {
-      float nv = xv[t];
-      if (p.mix) {
-        nv = outw[t] * v;
-#pragma unroll
-        for (int a = 0; a < S; ++a) nv = fmaf(mixv[a][t], xv[a], nv);
-        p.xs[t * plane + at] = nv;
+          for (int a = 0; a < S; ++a) nv = fmaf(mixv[a][t], xv[a][u], nv);
+        }
+        un = fmaf(inw[t], nv, un);
+        if (p.mix && d0 + 256 * u < p.D) p.xs[t * plane + row + dd[u]] = nv;
       }
-      u = fmaf(inw[t], nv, u);
+      if (p.next_in && d0 + 256 * u < p.D) p.u[row + dd[u]] = un;
     }
-    if (p.next_in) p.u[at] = u;
   }
 }
 
@@ -358,8 +372,16 @@ int hy_hc_update(const HyperUpdate& p, hipStream_t s) {
   if (p.mix && p.row_expert && (!p.row_w || !p.ident)) return -3;
   if ((p.next_in != nullptr) != (p.u != nullptr) || (!p.mix && !p.next_in)) return -4;
   if (p.M == 0) return 0;
+  const int nu = (p.D + 255) / 256;
   switch (p.S) {
-#define HC_CASE(N) case N: hc_update_kernel<N><<<p.M, 256, 0, s>>>(p); break
+#define HC_CASE(N)                                                                \
+  case N:                                                                         \
+    if (nu <= 1) hc_update_kernel<N, 1><<<p.M, 256, 0, s>>>(p);                   \
+    else if (nu <= 2) hc_update_kernel<N, 2><<<p.M, 256, 0, s>>>(p);              \
+    else if (nu <= 4) hc_update_kernel<N, 4><<<p.M, 256, 0, s>>>(p);              \
+    else if (nu <= 8 && N <= 4) hc_update_kernel<N, 8><<<p.M, 256, 0, s>>>(p);    \
+    else hc_update_kernel<N, 0><<<p.M, 256, 0, s>>>(p);                           \
+    break
     HC_CASE(1); HC_CASE(2); HC_CASE(3); HC_CASE(4); HC_CASE(5); HC_CASE(6); HC_CASE(7); HC_CASE(8);
 #undef HC_CASE
   }

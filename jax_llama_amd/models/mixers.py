@@ -226,7 +226,7 @@ class DenseFF:
         self.w_up, self.w_down, self.act = w_up, w_down, act
 
     def __call__(self, h: torch.Tensor, ctx: StepContext) -> FFOut:
-        return FFOut(hy.linear(hy.linear(h, self.w_up, act=self.act), self.w_down))
+        return FFOut(hy.ff_dense(h, self.w_up, self.w_down, self.act))
 
 
 class RoutedMoE:
@@ -495,9 +495,9 @@ class RotaryLatentAttention(LatentAttention):
         gate = proj[:, sp.q_rank + row:sp.q_rank + row + nh]
         s0 = ctx.cache.index if torch.is_tensor(ctx.slot0) else int(ctx.slot0)  # (host mirror of the slot)
         n = s0 + ctx.s
-        wide = row > hy.ATTN_MAX_HEAD
+        wide = row > hy.ATTN_MAX_KEY or rank > hy.ATTN_MAX_HEAD
         if wide and c.is_cuda and torch.cuda.is_current_stream_capturing():
-            raise NotImplementedError(f"latent attention: a cache row of {row} > {hy.ATTN_MAX_HEAD} in a captured step")
+            raise NotImplementedError(f"latent attention: a cache row of {rank} + {rot} in a captured step")
         if wide or (ctx.s > 1 and self.expands(ctx.s, n, c.dtype == torch.bfloat16)):
             # only the keys some query of the step can see are expanded: with a window and no kept first keys, the
             # scratch keys start at `first` and the step's slot is counted from there
@@ -579,7 +579,7 @@ class GroupedMoE:
                                               self.w_down, self.act)
         extra = None
         if self.shared_up is not None:
-            extra = hy.linear(hy.linear(hv, self.shared_up, act=self.act), self.shared_down)
+            extra = hy.ff_dense(hv, self.shared_up, self.shared_down, self.act)
         return MixtureOut(y, self.top, row_w, row_expert, self.experts, hv, extra)
 
 

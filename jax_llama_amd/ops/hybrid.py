@@ -44,8 +44,9 @@ import torch
 BF16 = torch.bfloat16
 F32 = torch.float32
 
-# widest key / value head the attention kernels take (csrc/hybrid/attn_bias.hip AB_MAX_DIM)
+# widest value head, and widest key head, the attention kernels take (csrc/hybrid/attn_bias.hip AB_MAX_VREG, AB_MAX_DIM)
 ATTN_MAX_HEAD = 512
+ATTN_MAX_KEY = 1024
 # epilogues of a row linear (csrc/hybrid/hybrid.h RowAct)
 ACT_NONE, ACT_RELU2, ACT_SWIGLU, ACT_CLAMP_GLU, ACT_SOFTCAP = 0, 1, 2, 3, 4
 
@@ -221,6 +222,26 @@ def linear(x, w: torch.Tensor, swiglu: bool = False, act: int = ACT_NONE, limit:
     ext().linear_rows(x, None, w, out, None, None, None, x.shape[0], int(act), float(limit), float(alpha), None, norm_w,
                       norm_eps)
     return out
+
+
+def ff_dense(x, w_up: torch.Tensor, w_down: torch.Tensor, act: int = ACT_RELU2) -> torch.Tensor:
+    """``act(x @ w_up^T) @ w_down^T`` with a one-accumulator activation. A prompt-sized bf16 batch runs both products on
+    the packed MFMA GEMM: it has no such epilogue, so the activation is applied by the kernel that rounds the hidden
+    activation to bf16 for the second product (a pass that product needs anyway). Otherwise the row linear with the
+    activation in its epilogue."""
+    if isinstance(x, RmsInput) and _gpu(w_up) and x.shape[0] >= PACKED_GEMM_MIN_M:
+        x = x.value()  # (the packed GEMM takes a normed activation, it does not norm it)
+    if (act in (ACT_NONE, ACT_RELU2) and _gpu(w_up) and not isinstance(x, RmsInput) and _use_packed_gemm(x, w_up)
+            and w_down.dtype == BF16 and w_down.shape[0] % 16 == 0 and w_down.shape[1] % 32 == 0
+            and (x.shape[0] * w_up.shape[0]) % 8 == 0):
+        from . import linear as packed_linear
+        xb = torch.empty(x.shape, dtype=BF16, device=x.device)
+        ext().cast_bf16(x, xb)
+        h = packed_linear(xb, _packed_weight(w_up), out_dtype=F32)
+        hb = torch.empty(h.shape, dtype=BF16, device=x.device)
+        ext().cast_bf16(h, hb, int(act))
+        return packed_linear(hb, _packed_weight(w_down), out_dtype=F32)
+    return linear(linear(x, w_up, act=act), w_down)
 
 
 def linear_add_(res: torch.Tensor, x, w: torch.Tensor) -> torch.Tensor:
@@ -467,9 +488,15 @@ def moe_grouped(x: torch.Tensor, z: torch.Tensor, correction: Optional[torch.Ten
         # expert-grouped over the sorted rows; identity experts sort behind the real ones, past the last offset the
         # linears look at
         e.route_grouped(z, correction, e_all, top, groups, keep, row_expert, row_tok, row_w, sort_tok, sort_dst, sort_w, offs)
+        # with bf16 weights the tiles read a bf16 copy of x and keep the hidden activation bf16 (the operands they would
+        # round to anyway): half the activation traffic of both products
         keep_bf16 = w_up.dtype == BF16 and r > GROUPED_GEMV_MAX_R
         h = torch.empty(r, f, dtype=BF16 if keep_bf16 else F32, device=dev)
-        e.linear_rows(x, sort_tok, w_up, h, None, offs, None, r, int(act), 0.0, 1.0, None, None, 0.0)
+        xa = x
+        if keep_bf16 and x.is_contiguous() and x.numel() % 8 == 0:
+            xa = torch.empty(x.shape, dtype=BF16, device=dev)
+            e.cast_bf16(x, xa)
+        e.linear_rows(xa, sort_tok, w_up, h, None, offs, None, r, int(act), 0.0, 1.0, None, None, 0.0)
         e.linear_rows(h, None, w_down, y, sort_dst, offs, None, r, ACT_NONE, 0.0, 1.0, None, None, 0.0)
     return y, row_expert, row_w
 

@@ -283,9 +283,37 @@ def besulix_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int,
                                     "logit_softcap": 30.0, "layers": ls})
 
 
+def zifisun_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int, layers: int, vocab: int,
+                 kv_rank: int = 448, window: int = 1024, experts: int = 8, identity: int = 2, top: int = 2,
+                 streams: int = 2):
+    """A Zifisun config whose layers have a LLaMA layer's sizes: latent-attention layers (``heads`` heads whose keys are
+    ``head_dim / 2`` plain + ``head_dim / 2`` rotated numbers, values of ``head_dim``, a latent of ``kv_rank`` so that a
+    cache row is ``kv_rank + head_dim / 2`` wide, a query latent of ``3 kv_rank / 2``) alternating with attention layers
+    (``heads`` / ``kv_heads`` heads of ``head_dim``, the first 64 keys kept), windows of ``window``; every layer with a
+    mixture of ``experts`` experts of ``ffn / 4`` plus ``identity`` identity experts in 5 groups of which 3 are kept,
+    ``top`` per token, and a shared expert of ``ffn / 2`` (the active width of the dense FFN at top 2); ``streams``
+    residual streams."""
+    from ..config import ZifisunConfig
+    half = head_dim // 2
+    lat = dict(heads=heads, dim=half, rot_dim=half, vdim=head_dim, kv_rank=kv_rank, q_rank=kv_rank * 3 // 2,
+               scale=head_dim ** -0.5, rot={"base": 1e4, "dims": half}, mask={"size": window})
+    att = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5,
+               mask={"size": window, "keep_first": 64})
+    total = experts + identity
+    groups = 5 if total % 5 == 0 else 1
+    moe = {"kind": "moe", "expert": {"ff": ffn // 4},
+           "router": {"experts": experts, "identity": identity, "top": top,
+                      "groups": {"count": groups, "keep": min(3, groups)}},
+           "shared": {"ff": ffn // 2}}
+    ls = [{"type": "attention", "mixer": dict(att), "mlp": moe} if i % 2 else
+          {"type": "latent_attention", "mixer": dict(lat), "mlp": moe} for i in range(layers)]
+    return ZifisunConfig.from_dict({"architecture": "Zifisun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "streams": streams, "layers": ls})
+
+
 def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: int = 64, batches=(1, 8),
                    families=("zavevik", "llama"), progress=lambda m: None) -> Dict[str, object]:
-    """Prefill and decode throughput of the layer-list families (Zavevik, Zasevik, Besulix) beside LLaMA at equal layer sizes
+    """Prefill and decode throughput of the layer-list families (Zavevik, Zasevik, Besulix, Zifisun) beside LLaMA at equal layer sizes
     (random weights, bf16, synthetic ids), all through the decode engine: ``prefill_tokens_per_sec`` of one warm ``prompt_len``-token prompt per row
     and hipGraph-replayed ``decode_ms_per_token`` over ``gen_len`` steps behind it."""
     from ..config import LLaMAConfig
@@ -305,6 +333,9 @@ def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: 
             elif family == "besulix":
                 from ..models.besulix import BesulixForCausalLM
                 model = BesulixForCausalLM(besulix_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
+            elif family == "zifisun":
+                from ..models.zifisun import ZifisunForCausalLM
+                model = ZifisunForCausalLM(zifisun_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
             else:
                 cfg = LLaMAConfig(vocab_size=sz["vocab"], hidden_size=sz["width"], intermediate_size=sz["ffn"],
                                   num_hidden_layers=sz["layers"], num_attention_heads=sz["heads"],

@@ -207,7 +207,7 @@ def _run_attn(w, mc, h, eps, device, portions, dtype=F32):
 LATENT_SHAPES = [  # heads, dim, rot_dim, vdim, rank, q_rank, window, keep_first, rot_dims
     (3, 16, 8, 24, 20, 28, 9, 0, None), (1, 8, 2, 72, 56, 8, 0, 0, None), (12, 8, 4, 8, 24, 16, 17, 5, 2),
     (70, 8, 2, 4, 16, 8, 64, 0, None), (2, 24, 16, 40, 64, 32, 1, 0, None), (2, 16, 16, 16, 200, 24, 23, 23, None),
-    (2, 16, 6, 16, 500, 24, 30, 2, 0)]
+    (2, 16, 6, 16, 500, 24, 30, 2, 0), (2, 16, 64, 16, 512, 24, 30, 0, None)]
 
 
 @pytest.mark.parametrize("device", DEVICES)
