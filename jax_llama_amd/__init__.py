@@ -2,7 +2,8 @@
 public API of LSaldyt/JAX_llama (reference ``jax_llama/__init__.py:4-10``), plus a model registry with a second
 family (Zavevik: gated delta rule + biased attention + table-routed experts) and a third (Zasevik: latent attention
 with a softmax sink + dense / score-routed feed-forwards) and a fourth (Besulix: matrix memories + block-local rotary
-attention beside a time-mix recurrence) on the same layer-list step function.
+attention beside a time-mix recurrence) and a fifth (Zifisun: windowed latent / normed attention, grouped routing with
+identity experts, several residual streams) on the same layer-list step function.
 
 Framework layer: PyTorch-ROCm. Hot path: hand-written HIP kernels (``csrc/kernels``).
 Multi-GPU: one process per GPU, RCCL + a custom xGMI all-reduce. Decode: hipGraph replay.
