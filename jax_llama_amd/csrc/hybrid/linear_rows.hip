@@ -336,7 +336,9 @@ constexpr int HY_GROUPED_GEMV_MAX_R = 64;
 // output columns at or below which a dense linear of any row count runs the GEMV
 constexpr int HY_SKINNY_MAX_N = 16;
 
-static bool lr_grouped(const RowLinear& p) { return p.offs && p.R <= HY_GROUPED_GEMV_MAX_R; }
+// (the GEMV forms read and write fp32: a bf16 activation copy or a bf16 output always takes the tiles)
+static bool lr_fp32_io(const RowLinear& p) { return !p.a_bf16 && !p.out_bf16; }
+static bool lr_grouped(const RowLinear& p) { return p.offs && p.R <= HY_GROUPED_GEMV_MAX_R && lr_fp32_io(p); }
 static bool lr_skinny(const RowLinear& p) {
   // a handful of output columns (a router): tiles would leave the chip empty, so any number of rows runs the GEMV, each
   // group of 8 rows streaming the few weight rows again
@@ -344,7 +346,7 @@ static bool lr_skinny(const RowLinear& p) {
          (p.R + HY_GEMV_MAX_R - 1) / HY_GEMV_MAX_R <= 65535;
 }
 bool hy_linear_rows_is_gemv(const RowLinear& p) {
-  return lr_grouped(p) || lr_skinny(p) || (p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert));
+  return lr_grouped(p) || lr_skinny(p) || (p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert) && lr_fp32_io(p));
 }
 
 int hy_linear_rows(const RowLinear& p, hipStream_t s) {

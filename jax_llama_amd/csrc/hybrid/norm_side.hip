@@ -368,7 +368,7 @@ __global__ void __launch_bounds__(256) hc_update_kernel(HyperUpdate p) {
 
 int hy_hc_update(const HyperUpdate& p, hipStream_t s) {
   if (p.S < 1 || p.S > 8 || p.M < 0 || p.D < 1 || !p.xs) return -1;
-  if (p.mix && (!p.out_w || !p.y || p.nsum < 1 || p.nsum > 16)) return -2;
+  if (p.mix && (!p.out_w || !p.y || p.nsum < 1)) return -2;
   if (p.mix && p.row_expert && (!p.row_w || !p.ident)) return -3;
   if ((p.next_in != nullptr) != (p.u != nullptr) || (!p.mix && !p.next_in)) return -4;
   if (p.M == 0) return 0;

@@ -267,6 +267,19 @@ def test_attention_at_the_mfma_head_sizes(device, dtype):
         assert err(_run_latent(w, mc, h, eps, device, [100, 2, 147, 1, 50], dtype, form), ref) < lim, form
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_short_expanded_portions_in_bfloat16(device):
+    """One head and portions of a few dozen tokens in the expanded form with bf16 caches: the per-head maps of the cached
+    rows have fewer rows than one tile (the cache is a bf16 operand: no GEMV form reads it)."""
+    mc = _lat(1, 16, 8, 24, 40, 16, 0.3, window=30, base=100.0)
+    t, d, eps = 45, 48, 1e-6
+    g = torch.Generator().manual_seed(4)
+    w = {k: v.to(BF16).float() for k, v in _latent_weights(g, mc, d).items()}
+    h = torch.randn(t, d, generator=g).to(BF16).float()
+    ref = oz.latent_attention(w, "m.", mc, h.double().numpy(), eps)
+    assert err(_run_latent(w, mc, h, eps, device, [20, 3, 2, 17, 3], BF16, "expanded"), ref) < 3e-2
+
+
 def _point_at(wq, key):
     """An input whose projection by ``wq [n, d]`` (n <= d) is ``key``: the least-squares solution."""
     return np.linalg.lstsq(wq, key, rcond=None)[0]
