@@ -89,7 +89,7 @@ int hy_route_grouped(const float* z, int ldz, const float* correction, int M, in
 // at once from the old ones:   xs[t][m] <- sum_s mix[s * S + t] xs[s][m] + out_w[t] * v[m],
 //   v[m] = sum_{c < nsum} w_c y[m * nsum + c] (+ extra[m]),  w_c = row_w ? row_w[m * nsum + c] : 1;
 // with row_expert, a row whose expert is >= n_real is an identity expert: it adds w_c * ident[m] and its y row is not read.
-// With next_in != nullptr: u[m] = sum_t next_in[t] xs[t][m] of the (new) streams. mix == nullptr: only u. S <= 8.
+// With next_in != nullptr: u[m] = sum_t next_in[t] xs[t][m] of the (new) streams. mix == nullptr: only u. S <= 16.
 struct HyperUpdate {
   float* xs;
   int S, M, D;

@@ -367,7 +367,7 @@ __global__ void __launch_bounds__(256) hc_update_kernel(HyperUpdate p) {
 }
 
 int hy_hc_update(const HyperUpdate& p, hipStream_t s) {
-  if (p.S < 1 || p.S > 8 || p.M < 0 || p.D < 1 || !p.xs) return -1;
+  if (p.S < 1 || p.S > 16 || p.M < 0 || p.D < 1 || !p.xs) return -1;
   if (p.mix && (!p.out_w || !p.y || p.nsum < 1)) return -2;
   if (p.mix && p.row_expert && (!p.row_w || !p.ident)) return -3;
   if ((p.next_in != nullptr) != (p.u != nullptr) || (!p.mix && !p.next_in)) return -4;
@@ -384,6 +384,9 @@ int hy_hc_update(const HyperUpdate& p, hipStream_t s) {
     break
     HC_CASE(1); HC_CASE(2); HC_CASE(3); HC_CASE(4); HC_CASE(5); HC_CASE(6); HC_CASE(7); HC_CASE(8);
 #undef HC_CASE
+#define HC_WIDE(N) case N: hc_update_kernel<N, 0><<<p.M, 256, 0, s>>>(p); break  // (many streams: a column at a time)
+    HC_WIDE(9); HC_WIDE(10); HC_WIDE(11); HC_WIDE(12); HC_WIDE(13); HC_WIDE(14); HC_WIDE(15); HC_WIDE(16);
+#undef HC_WIDE
   }
   JLA_CHECK_LAUNCH();
   return 0;

@@ -447,11 +447,12 @@ class RotaryLatentAttention(LatentAttention):
 
     def __init__(self, layer_idx: int, spec, eps: float, w_in: torch.Tensor, dq_norm: torch.Tensor, w_uq: torch.Tensor,
                  dkv_norm: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, freq: Optional[torch.Tensor],
-                 w_o: torch.Tensor):
+                 w_o: torch.Tensor, gated: bool = True):
         self.i = layer_idx
+        self.gated = gated        # whether w_in ends with one gate row per head
         self.spec = spec
         self.eps = eps
-        self.w_in = w_in          # [q_rank + kv_rank + rot_dim + H, D]: query latent, key / value latent, rotated key, gates
+        self.w_in = w_in          # [q_rank + kv_rank + rot_dim (+ H), D]: query latent, key / value latent, rotated key, gates
         self.dq_norm, self.dkv_norm = dq_norm, dkv_norm  # fp32 [q_rank], [kv_rank]
         self.w_uq = w_uq          # [H (dim + rot_dim), q_rank]
         self.freq = freq          # float64 [rot_dims / 2] or None
@@ -492,7 +493,7 @@ class RotaryLatentAttention(LatentAttention):
         q = hy.linear(cq, self.w_uq)
         if self.freq is not None:
             hy.rotate_heads(q, ctx.positions, self.freq, nh, out=q, offset=sp.dim, interleaved=True)
-        gate = proj[:, sp.q_rank + row:sp.q_rank + row + nh]
+        gate = proj[:, sp.q_rank + row:sp.q_rank + row + nh] if self.gated else None
         s0 = ctx.cache.index if torch.is_tensor(ctx.slot0) else int(ctx.slot0)  # (host mirror of the slot)
         n = s0 + ctx.s
         wide = row > hy.ATTN_MAX_KEY or rank > hy.ATTN_MAX_HEAD

@@ -147,8 +147,10 @@ class ZifisunForCausalLM(LayerListLM):
                 w_uk = sd[p + "mix.uk"].reshape(m.heads, m.dim, m.kv_rank).to(dev, wdt)
                 w_uv = sd[p + "mix.uv"].reshape(m.heads, m.vdim, m.kv_rank).to(dev, wdt).contiguous()
                 freq = hy.rotary_freqs(m.rot_base, m.rot_dims, dev) if m.rot_dims else None
-                args = (m, eps, mat(p + "mix.dq", p + "mix.dkv", p + "mix.g"), f32(p + "mix.dq.norm"), mat(p + "mix.uq"),
-                        f32(p + "mix.dkv.norm"), w_uk, w_uv, freq, mat(p + "mix.o"))
+                gated = p + "mix.g" in sd
+                names = [p + "mix.dq", p + "mix.dkv"] + ([p + "mix.g"] if gated else [])
+                args = (m, eps, mat(*names), f32(p + "mix.dq.norm"), mat(p + "mix.uq"), f32(p + "mix.dkv.norm"), w_uk, w_uv,
+                        freq, mat(p + "mix.o"), gated)
                 make = RotaryLatentAttention
             elif isinstance(m, NormedAttentionSpec):
                 want(p + "mix.q", (m.heads * m.dim, c.hidden_size))

@@ -207,7 +207,7 @@ def _run_attn(w, mc, h, eps, device, portions, dtype=F32):
 LATENT_SHAPES = [  # heads, dim, rot_dim, vdim, rank, q_rank, window, keep_first, rot_dims
     (3, 16, 8, 24, 20, 28, 9, 0, None), (1, 8, 2, 72, 56, 8, 0, 0, None), (12, 8, 4, 8, 24, 16, 17, 5, 2),
     (70, 8, 2, 4, 16, 8, 64, 0, None), (2, 24, 16, 40, 64, 32, 1, 0, None), (2, 16, 16, 16, 200, 24, 23, 23, None),
-    (2, 16, 6, 16, 500, 24, 30, 2, 0), (2, 16, 64, 16, 512, 24, 30, 0, None)]
+    (2, 16, 6, 16, 500, 24, 30, 2, 0), (2, 16, 64, 16, 512, 24, 30, 0, None), (2, 16, 8, 16, 520, 24, 30, 0, None)]
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -480,7 +480,8 @@ def test_group_limit_and_selection_bias_change_the_choice():
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("streams,m,d", [(1, 3, 40), (2, 1, 24), (3, 70, 40), (4, 5, 300), (8, 2, 1030)])
+@pytest.mark.parametrize("streams,m,d", [(1, 3, 40), (2, 1, 24), (3, 70, 40), (4, 5, 300), (8, 2, 1030), (11, 3, 40),
+                                         (5, 2, 2100), (2, 3, 2048)])
 def test_stream_update(device, streams, m, d):
     """The hyper-connection kernels alone: the read (a weighted sum of the streams) and the write (all streams at once
     from the old ones, the mixing matrix indexed [from, to], which a transposed matrix would get wrong)."""
