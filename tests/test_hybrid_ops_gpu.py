@@ -299,3 +299,81 @@ def test_moe_routed_norms_its_input(dt, m, top):
     got = hy.moe_routed(hy.RmsInput(x.to(DEV), gain.to(DEV), 1e-5), z.to(DEV), top, w_gu.to(DEV), w_down.to(DEV),
                         hy.ACT_CLAMP_GLU, 0.9, 1.702)
     _close(got, ref, 2e-5 if dt == torch.float32 else 4e-3, "routed moe, fused input norm")
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("shape", [  # every attention kernel: plain / fast / shared-latent decode, plain / MFMA prefill
+    dict(b=2, s=1, s0=300, h=4, g=2, dim=48, vdim=40), dict(b=1, s=1, s0=700, h=4, g=1, dim=64, vdim=128),
+    dict(b=2, s=1, s0=333, h=6, g=1, dim=264, vdim=232, shared=True), dict(b=1, s=1, s0=90, h=3, g=1, dim=96, vdim=64, shared=True),
+    dict(b=1, s=70, s0=131, h=4, g=2, dim=48, vdim=40), dict(b=2, s=150, s0=77, h=4, g=2, dim=128, vdim=64),
+    dict(b=1, s=100, s0=250, h=2, g=1, dim=96, vdim=64, shared=True)])
+@pytest.mark.parametrize("window,keep", [(1, 0), (37, 0), (64, 5), (100, 130), (1000, 3)])
+def test_attention_windows_gates_and_wide_value_rows(dt, shape, window, keep):
+    """Sliding windows with kept first keys, the gate per (token, head) and values that are the leading columns of the
+    key rows (one shared cache), in every attention kernel against the CPU op."""
+    b, s, s0, h, g, dim, vdim = (shape[k] for k in ("b", "s", "s0", "h", "g", "dim", "vdim"))
+    t = s0 + s + 3
+    q = _rand(b, s, h, dim, std=0.5)
+    kc = _rand(b, g, t, dim, dt=dt)
+    vc = kc if shape.get("shared") else _rand(b, g, t, vdim, dt=dt)
+    gate = _rand(b * s, h + 2)[:, 1:h + 1]  # a column view of a wider projection
+    kw = dict(window=window, keep_first=keep, vdim=vdim if shape.get("shared") else None)
+    kg = kc.to(DEV)
+    vg = kg if shape.get("shared") else vc.to(DEV)
+    gg = gate.to(DEV)
+    for gt, gr in ((gg, gate), (None, None)):
+        ref = hy.attn_bias(q, kc, vc, s0, dim ** -0.5, gate=gr, **kw)
+        got = hy.attn_bias(q.to(DEV), kg, vg, s0, dim ** -0.5, gate=gt, **kw)
+        # (the MFMA prefill rounds q to bf16 for the score product like any other matrix operand)
+        mma = dt == torch.bfloat16 and s > 1 and dim in (64, 128) and vdim in (64, 128) and not shape.get("shared")
+        _close(got, ref, 2e-2 if mma else 2e-5, f"window {window} keep {keep}")
+    with pytest.raises(ValueError):
+        hy.attn_bias(q, kc, vc, s0, 1.0, chunk=8, window=4)
+
+
+@pytest.mark.parametrize("m,e,top,groups,keep", [(1, 10, 2, 5, 3), (7, 1, 1, 1, 1), (40, 12, 4, 4, 2), (300, 64, 5, 8, 3),
+                                                 (9, 70, 6, 7, 1), (65, 1000, 8, 10, 4), (33, 20, 4, 4, 3)])
+@pytest.mark.parametrize("biased", [True, False])
+def test_route_grouped(m, e, top, groups, keep, biased):
+    """The grouped softmax router's record (one-pass form up to 64 experts, round-based beyond): the chosen set and the
+    weights of the CPU op, and an expert-sorted order that is a permutation of the rows with the right offsets."""
+    top = min(top, keep * (e // groups))
+    z = _rand(m, e + 3, std=2.0)[:, :e]
+    corr = _rand(e, std=0.05) if biased else None
+    ex_ref, w_ref = hy.route_grouped(z, corr, top, groups, keep)
+    r = m * top
+    idx = torch.empty(4 * r + e + 1, dtype=torch.int32, device=DEV)
+    wts = torch.empty(2 * r, dtype=torch.float32, device=DEV)
+    hy.ext().route_grouped(z.to(DEV), corr.to(DEV) if biased else None, e, top, groups, keep, idx[:r], idx[r:2 * r], wts[:r],
+                           idx[2 * r:3 * r], idx[3 * r:4 * r], wts[r:], idx[4 * r:])
+    ex, tok, stok, sdst, offs = (x.cpu() for x in (idx[:r], idx[r:2 * r], idx[2 * r:3 * r], idx[3 * r:4 * r], idx[4 * r:]))
+    order = torch.argsort(ex.reshape(m, top), 1)
+    assert torch.equal(torch.gather(ex.reshape(m, top), 1, order).long(), torch.sort(ex_ref.reshape(m, top), 1).values)
+    by_expert = torch.gather(w_ref.reshape(m, top), 1, torch.argsort(ex_ref.reshape(m, top), 1))
+    _close(torch.gather(wts[:r].cpu().reshape(m, top), 1, order), by_expert, 1e-5, "weights")
+    assert torch.equal(tok, torch.arange(m, dtype=torch.int32).repeat_interleave(top))
+    assert int(offs[0]) == 0 and int(offs[e]) == r and torch.equal(torch.sort(sdst).values.long(), torch.arange(r))
+    assert torch.equal(ex[sdst.long()], torch.sort(ex).values) and torch.equal(stok, tok[sdst.long()])
+    _close(wts[r:], wts[:r][sdst.long().to(DEV)], 0.0, "sorted weights")
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("m,experts,identity,top", [(1, 4, 2, 3), (2, 6, 2, 4), (20, 3, 5, 2), (150, 8, 2, 2), (700, 2, 1, 1)])
+def test_moe_grouped_and_the_stream_update(dt, m, experts, identity, top):
+    """Experts with identity experts behind them on all three linear paths, summed by the stream update, against the CPU
+    ops; the feed-forward of a prompt on the packed GEMM against the row linear."""
+    d, ff, streams = 64, 96, 3
+    x = _rand(m, d)
+    z = _rand(m, experts + identity, std=2.0)
+    w_up, w_down = _rand(experts, ff, d, dt=dt, std=d ** -0.5), _rand(experts, d, ff, dt=dt, std=ff ** -0.5)
+    y, ex, wt = hy.moe_grouped(x, z, None, top, 1, 1, w_up, w_down)
+    yg, exg, wtg = hy.moe_grouped(x.to(DEV), z.to(DEV), None, top, 1, 1, w_up.to(DEV), w_down.to(DEV))
+    xs = _rand(streams, m, d)
+    mix, ow, nxt, extra = _rand(streams, streams), _rand(streams), _rand(streams), _rand(m, d)
+    xg = xs.to(DEV).clone()
+    u = hy.hc_update_(xs, mix, ow, y, top, wt, ex, experts, x, extra, next_in=nxt)
+    ug = hy.hc_update_(xg, mix.to(DEV), ow.to(DEV), yg, top, wtg, exg, experts, x.to(DEV), extra.to(DEV), next_in=nxt.to(DEV))
+    _close(xg, xs, 5e-5, "streams")
+    _close(ug, u, 5e-5, "next input")
+    s_up, s_down = _rand(ff, d, dt=dt, std=d ** -0.5), _rand(d, ff, dt=dt, std=ff ** -0.5)
+    _close(hy.ff_dense(x.to(DEV), s_up.to(DEV), s_down.to(DEV)), hy.ff_dense(x, s_up, s_down), 2e-5, "one-accumulator FF")
